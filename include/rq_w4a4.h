@@ -1,0 +1,131 @@
+/*
+ * C ABI of the MI355X (gfx950) implementation of ruquant's W4A4 / W4A4H MUL_MAT.
+ *
+ * Plain pointers and sizes only. Every device pointer is memory of the current HIP device; `stream` is a
+ * hipStream_t passed as void* (the reference's Rust host passes its stream the same way,
+ * src/kernels.rs:14). Citations "P:n" are lines of patches/llama.cpp-ruquant.patch in the reference.
+ *
+ * Life cycle of one weight tensor, mirroring the reference's first-use / steady-state split
+ * (P:2027-2075, P:295-299):
+ *   first use   (may synchronize, must not be captured in a graph):
+ *       read block 0's header on the host -> rq_w4a4_resolve_clip / rq_w4a4_rot_check;
+ *       rq_w4a4_prepare() rewrites the 144-byte blocks into the streaming layout, OUT OF PLACE
+ *       (the reference repacks in place and leaves the tensor unreadable as blocks; this does not).
+ *   steady state (no allocation, no synchronization, no host reads: safe inside HIP graph capture):
+ *       rq_w4a4_mul_mat() on the prepared weights.
+ *
+ * Return values: 0 = success; > 0 = a hipError_t; < 0 = one of the RQ_E_* codes below.
+ */
+#ifndef RQ_W4A4_H
+#define RQ_W4A4_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RQ_TYPE_W4A4   44   /* GGML_TYPE_W4A4  (P:10) */
+#define RQ_TYPE_W4A4H  45   /* GGML_TYPE_W4A4H (P:11) */
+#define RQ_TYPE_A4     46   /* GGML_TYPE_A4    (P:12) */
+#define RQ_TYPE_A4H    47   /* GGML_TYPE_A4H   (P:13) */
+
+#define RQ_BLOCK_CODES 256  /* QK_W4A4 (P:38) */
+#define RQ_BLOCK_BYTES 144  /* sizeof(block_w4a4) (P:44-50) */
+#define RQ_MAX_K       32768 /* QK_W4A4 * RQ_MAX_BLOCKS (P:1748, P:1982) */
+
+#define RQ_E_UNSUPPORTED  (-1)  /* shape/type the op does not take (the reference says so via supports_op) */
+#define RQ_E_WORKSPACE    (-2)  /* workspace or prepared buffer too small or misaligned */
+#define RQ_E_ARGUMENT     (-3)  /* null pointer, bad clip, bad rotation length */
+
+typedef void *rq_stream_t;
+
+/* block_w4a4 as stored in a W4A4 / W4A4H tensor (P:44-50). */
+typedef struct {
+    float    d;       /* row unit s_w, repeated in every block of the row */
+    int32_t  sum;     /* 1<<30 | k, or 3<<29 | k0 | k1<<4 | k2<<8 | k3<<12, or the legacy row code sum (k = 1) */
+    int32_t  pad[2];  /* pad[0] = row length (W4A4) / Hadamard length (W4A4H); pad[1] = clip as float bits */
+    uint32_t qs[32];  /* element 8w+j in bits [4j+3:4j] of qs[w] */
+} rq_block_w4a4;
+
+/* ---- host-side queries (no GPU work) -------------------------------------------------------------- */
+
+/* Replaces ggml_cuda_rq_w4a4_supported (P:1977-1994): 1 if rq_w4a4_mul_mat takes this problem.
+ * src1 / dst must be fp32 with element stride 4; ldx_bytes / ldy_bytes are their row strides in bytes. */
+int rq_w4a4_supported(int type, int64_t K, int64_t N, int64_t M, int64_t ldx_bytes, int64_t ldy_bytes);
+
+/* Replaces ggml_rq_hadamard_factor (P:2419-2430). Returns 1 and n = p * m, else 0. */
+int rq_w4a4_hadamard_factor(int64_t n, int *p, int *m);
+
+/* Replaces ggml_rq_act_clip_for(ggml_rq_tensor_clip(blocks), had) (P:2590-2606): RQ_ACT_CLIP[_H] from the
+ * environment (read once per process, as the reference does), else the header's pad[1], else 1.
+ * host_block0 points at the first 16 bytes (or more) of the tensor, in host memory. */
+float rq_w4a4_resolve_clip(const void *host_block0, int type);
+
+/* Replaces ggml_rq_tensor_rot / ggml_rq_rot_check (P:2608-2620): the Hadamard length in pad[0] if it is
+ * positive, divides K and factors; -1 where the reference aborts. For RQ_TYPE_W4A4 returns 0. */
+int64_t rq_w4a4_tensor_rot(const void *host_block0, int type, int64_t K);
+
+/* Replaces ggml_rq_act_group (P:2623-2631): 64, or RQ_ACT_GROUP = 128 / 256 (read once). */
+int rq_w4a4_act_group(void);
+
+/* ---- first use ------------------------------------------------------------------------------------ */
+
+/* Bytes of the prepared (streaming) form of an N x K weight; a multiple of 256. */
+size_t rq_w4a4_prepared_bytes(int64_t K, int64_t N);
+
+/* Replaces rq_repack_once (P:2046-2075), out of place: reads N rows of K/256 blocks at w_blocks_dev, writes
+ * prepared_dev (256-byte aligned, rq_w4a4_prepared_bytes). Asynchronous on `stream`; the input is not
+ * modified and may be freed once the stream has passed this call. */
+int rq_w4a4_prepare(const void *w_blocks_dev, int64_t K, int64_t N,
+                    void *prepared_dev, size_t prepared_bytes, rq_stream_t stream);
+
+/* ---- steady state --------------------------------------------------------------------------------- */
+
+/* Scratch the op needs for this problem (quantized activations, multipliers, split-K sums); a multiple of
+ * 256. The reference takes the same buffers from the backend pool (P:2106-2109, P:2232-2235). */
+size_t rq_w4a4_workspace_bytes(int type, int64_t K, int64_t N, int64_t M);
+
+/* Replaces ggml_cuda_mul_mat_rq_w4a4 (P:2341-2347, rq_mul_mat P:2145-2338):
+ *   y[t][n] = W[n] . x[t], t < M, n < N, bit-identical to ggml_vec_dot_w4a4_a4 (P:148-177) on activations
+ *   quantized by quantize_row_a4_clip / quantize_row_a4h_clip_n (P:2639-2679, P:2728-2736).
+ * x_dev: M rows of K floats, row stride ldx floats (ldx * 4 a multiple of 16); y_dev: M rows of N floats,
+ * row stride ldy floats. clip > 0 (rq_w4a4_resolve_clip); n_rot = rq_w4a4_tensor_rot (ignored for W4A4).
+ * workspace_dev: 256-byte aligned, at least rq_w4a4_workspace_bytes; its contents need not be preserved
+ * between calls, and two calls that overlap in time must not share it. */
+int rq_w4a4_mul_mat(int type, const void *prepared_dev, int64_t K, int64_t N,
+                    const float *x_dev, int64_t ldx, int64_t M,
+                    float *y_dev, int64_t ldy,
+                    float clip, int64_t n_rot,
+                    void *workspace_dev, size_t workspace_bytes, rq_stream_t stream);
+
+/* Replaces ggml_cuda_mul_mat_rq_w4a4_fused (P:2371-2380): n <= 3 weights of one type, K, clip and rotation
+ * length against the same x (q/k/v, gate/up): one activation transform, then one product per weight.
+ * workspace: rq_w4a4_workspace_bytes for the largest N. */
+int rq_w4a4_mul_mat_fused(int type, int n, const void *const *prepared_dev, int64_t K, const int64_t *N,
+                          const float *x_dev, int64_t ldx, int64_t M,
+                          float *const *y_dev, const int64_t *ldy,
+                          float clip, int64_t n_rot,
+                          void *workspace_dev, size_t workspace_bytes, rq_stream_t stream);
+
+/* ---- the activation side on its own (the A4 / A4H from_float of the CPU type traits, P:71-88) ------- */
+
+/* Replaces ggml_rq_hadamard per rotation block (P:2450-2485, P:2697-2699): out[t] = x[t] diag(H, H, ...),
+ * M rows of K floats, each n_rot-long block rotated; out row stride ldo floats. */
+int rq_w4a4_hadamard(const float *x_dev, int64_t ldx, int64_t M, int64_t K, int64_t n_rot,
+                     float *out_dev, int64_t ldo, rq_stream_t stream);
+
+/* Replaces quantize_row_a4_clip / quantize_row_a4h_clip_n (P:2639-2679, P:2728-2736): writes M rows of
+ * K/256 activation blocks in the reference's A4 / A4H storage layout (byte-identical to the CPU's work
+ * buffer). type is RQ_TYPE_A4 (no rotation) or RQ_TYPE_A4H. */
+int rq_w4a4_quantize_act(int type, const float *x_dev, int64_t ldx, int64_t M, int64_t K,
+                         float clip, int64_t n_rot, void *blocks_dev, rq_stream_t stream);
+
+/* Library version, for the host binding to check. */
+int rq_w4a4_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

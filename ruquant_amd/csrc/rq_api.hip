@@ -1,0 +1,308 @@
+// extern "C" layer of the gfx950 W4A4 / W4A4H MUL_MAT library: argument checks, clip / rotation-length
+// resolution, workspace carving and the choice between the GEMV and the MFMA GEMM.
+#include "rq_common.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+namespace rq {
+
+// same search as the reference's ggml_rq_hadamard_factor (reference patch lines 2419-2430): smallest p first
+bool hadamard_factor(int64_t n, int &p, int &m) {
+    for (int cand = 1; cand <= 128 && cand <= n; ++cand) {
+        if (cand > 1) {
+            if (cand % 4 != 0 || (cand - 1) % 4 != 3) continue;
+            bool prime = cand - 1 >= 2;
+            for (int d = 2; d * d <= cand - 1; ++d) {
+                if ((cand - 1) % d == 0) {
+                    prime = false;
+                    break;
+                }
+            }
+            if (!prime) continue;
+        }
+        if (n % cand != 0) continue;
+        const int64_t rest = n / cand;
+        if (rest & (rest - 1)) continue;
+        p = cand;
+        m = (int) rest;
+        return true;
+    }
+    return false;
+}
+
+namespace {
+
+// Environment switches are read once per process, as the reference's function-local statics do
+// (reference patch lines 2590-2600, 2623-2631).
+struct Env {
+    float clip[2];   // RQ_ACT_CLIP, RQ_ACT_CLIP_H (falls back to the former); -1 = unset
+    int   act_group;
+    int   gemm_min;  // smallest token count that takes the MFMA GEMM
+    Env() {
+        const char *e = getenv("RQ_ACT_CLIP");
+        const char *eh = getenv("RQ_ACT_CLIP_H");
+        clip[0] = e ? (float) atof(e) : -1.0f;
+        clip[1] = eh ? (float) atof(eh) : clip[0];
+        const char *g = getenv("RQ_ACT_GROUP");
+        const int v = g ? atoi(g) : 64;
+        act_group = v == 128 || v == 256 ? v : 64;
+        const char *gm = getenv("RQ_GEMM_MIN");
+        gemm_min = gm ? atoi(gm) : 33;
+        if (gemm_min < 1) gemm_min = 1;
+    }
+};
+
+const Env &env() {
+    static const Env e;
+    return e;
+}
+
+bool is_w_type(int type) { return type == RQ_TYPE_W4A4 || type == RQ_TYPE_W4A4H; }
+
+bool shape_ok(int type, int64_t K, int64_t N, int64_t M) {
+    if (!is_w_type(type)) return false;
+    if (K <= 0 || K % RQ_BLOCK_CODES != 0 || K > RQ_MAX_K) return false;
+    if (N <= 0 || N > (int64_t) 1 << 24) return false;
+    if (M < 0 || M > (int64_t) 1 << 24) return false;
+    return true;
+}
+
+// rotation parameters of one call; returns false where the reference aborts (reference patch lines 2612-2620)
+bool rotation_of(int type, int64_t K, int64_t n_rot, int &p, int &m) {
+    p = 1;
+    m = 1;
+    if (type != RQ_TYPE_W4A4H) return true;
+    if (n_rot <= 0 || n_rot > K || K % n_rot != 0) return false;
+    return hadamard_factor(n_rot, p, m);
+}
+
+bool use_gemm(int64_t M) { return M >= env().gemm_min; }
+
+int run_products(int type, int n, const void *const *prepared, int64_t K, const int64_t *N, const float *x,
+                 int64_t ldx, int64_t M, float *const *y, const int64_t *ldy, float clip, int64_t n_rot, void *ws,
+                 size_t ws_bytes, hipStream_t stream) {
+    if (n < 1 || n > 3 || !prepared || !N || !y || !ldy || !x || !ws) return RQ_E_ARGUMENT;
+    int64_t Nmax = 0;
+    for (int i = 0; i < n; ++i) {
+        if (!shape_ok(type, K, N[i], M)) return RQ_E_UNSUPPORTED;
+        if (!prepared[i] || !y[i] || ldy[i] < N[i]) return RQ_E_ARGUMENT;
+        if ((reinterpret_cast<uintptr_t>(prepared[i]) & 255) != 0) return RQ_E_WORKSPACE;
+        if (N[i] > Nmax) Nmax = N[i];
+    }
+    if (env().act_group != 64) return RQ_E_UNSUPPORTED;
+    if (!(clip > 0.0f) || !isfinite(clip)) return RQ_E_ARGUMENT;
+    if (ldx < K || (ldx * 4) % 16 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0) return RQ_E_ARGUMENT;
+    int p, m;
+    if (!rotation_of(type, K, n_rot, p, m)) return RQ_E_ARGUMENT;
+    if (M == 0) return 0;
+
+    const WorkspaceLayout W = workspace_layout(K, Nmax, M);
+    if (ws_bytes < W.bytes || (reinterpret_cast<uintptr_t>(ws) & 255) != 0) return RQ_E_WORKSPACE;
+    uint8_t *wsb = reinterpret_cast<uint8_t *>(ws);
+
+    const bool gemm = use_gemm(M);
+    RotQuantArgs q;
+    memset(&q, 0, sizeof q);
+    q.x = x;
+    q.ldx = ldx;
+    q.M = (int) M;
+    q.K = (int) K;
+    q.rotate = type == RQ_TYPE_W4A4H;
+    q.n_rot = (int) (q.rotate ? n_rot : K);
+    q.p = p;
+    q.m = m;
+    q.scale = 1.0f / sqrtf((float) q.n_rot);
+    q.clip = clip;
+    q.mode = gemm ? kActI8 : kActQ4;
+    q.u = reinterpret_cast<float *>(wsb + W.off_u);
+    q.act = reinterpret_cast<uint32_t *>(wsb + W.off_act);
+    q.mz = wsb + W.off_mz;
+    q.Mp = (int) W.Mp;
+    if (!gemm) {
+        q.zero_ptr = reinterpret_cast<int32_t *>(wsb + W.off_tot);
+        q.zero_ints = (int64_t) ((W.bytes - W.off_tot) / sizeof(int32_t));
+    }
+    hipError_t e = launch_rotate_quant(q, stream);
+    if (e != hipSuccess) return (int) e;
+
+    for (int i = 0; i < n; ++i) {
+        const PreparedLayout L = prepared_layout(K, N[i]);
+        if (gemm) {
+            GemmArgs g;
+            g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
+            g.L = L;
+            g.act8 = wsb + W.off_act;
+            g.m8 = wsb + W.off_mz;
+            g.u = q.u;
+            g.y = y[i];
+            g.ldy = ldy[i];
+            g.M = (int) M;
+            g.Mp = (int) W.Mp;
+            e = launch_gemm(g, stream);
+            if (e != hipSuccess) return (int) e;
+        } else {
+            for (int c = 0; c < W.chunks; ++c) {
+                GemvArgs g;
+                g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
+                g.L = L;
+                g.act = q.act + (size_t) c * L.ng * kGemvTokens * 8;
+                g.mz = reinterpret_cast<const int32_t *>(wsb + W.off_mz) + (size_t) c * L.ng * kGemvTokens;
+                g.u = q.u + c * kGemvTokens;
+                g.y = y[i] + (int64_t) c * kGemvTokens * ldy[i];
+                g.ldy = ldy[i];
+                g.T = (int) (M - (int64_t) c * kGemvTokens < kGemvTokens ? M - (int64_t) c * kGemvTokens : kGemvTokens);
+                g.tot = reinterpret_cast<int32_t *>(wsb + W.off_tot);
+                g.cnt = reinterpret_cast<int32_t *>(wsb + W.off_cnt);
+                e = launch_gemv(g, stream);
+                if (e != hipSuccess) return (int) e;
+            }
+        }
+    }
+    return 0;
+}
+
+}  // namespace
+}  // namespace rq
+
+using namespace rq;
+
+extern "C" {
+
+int rq_w4a4_abi_version(void) { return 1; }
+
+int rq_w4a4_hadamard_factor(int64_t n, int *p, int *m) {
+    int pp = 0, mm = 0;
+    if (n <= 0 || !hadamard_factor(n, pp, mm)) return 0;
+    if (p) *p = pp;
+    if (m) *m = mm;
+    return 1;
+}
+
+int rq_w4a4_act_group(void) { return env().act_group; }
+
+int rq_w4a4_supported(int type, int64_t K, int64_t N, int64_t M, int64_t ldx_bytes, int64_t ldy_bytes) {
+    if (!shape_ok(type, K, N, M)) return 0;
+    if (ldx_bytes % 16 != 0 || ldx_bytes < K * 4) return 0;
+    if (ldy_bytes % 4 != 0 || ldy_bytes < N * 4) return 0;
+    if (env().act_group != 64) return 0;
+    if (type == RQ_TYPE_W4A4H) {
+        int p, m;
+        if (!hadamard_factor(K, p, m)) return 0;  // the whole-row rotation must exist (reference line 1986)
+    }
+    return 1;
+}
+
+float rq_w4a4_resolve_clip(const void *host_block0, int type) {
+    float tensor_clip = 0.0f;
+    if (host_block0) memcpy(&tensor_clip, reinterpret_cast<const char *>(host_block0) + 12, sizeof tensor_clip);
+    const float e = env().clip[type == RQ_TYPE_W4A4H || type == RQ_TYPE_A4H ? 1 : 0];
+    return e > 0.0f ? e : tensor_clip > 0.0f ? tensor_clip : 1.0f;
+}
+
+int64_t rq_w4a4_tensor_rot(const void *host_block0, int type, int64_t K) {
+    if (type != RQ_TYPE_W4A4H && type != RQ_TYPE_A4H) return 0;
+    if (!host_block0) return -1;
+    int32_t n = 0;
+    memcpy(&n, reinterpret_cast<const char *>(host_block0) + 8, sizeof n);
+    int p, m;
+    if (n <= 0 || K % n != 0 || !hadamard_factor(n, p, m)) return -1;
+    return n;
+}
+
+size_t rq_w4a4_prepared_bytes(int64_t K, int64_t N) {
+    if (K <= 0 || K % RQ_BLOCK_CODES != 0 || K > RQ_MAX_K || N <= 0) return 0;
+    return prepared_layout(K, N).bytes;
+}
+
+int rq_w4a4_prepare(const void *w_blocks_dev, int64_t K, int64_t N, void *prepared_dev, size_t prepared_bytes,
+                    rq_stream_t stream) {
+    if (!w_blocks_dev || !prepared_dev) return RQ_E_ARGUMENT;
+    if (K <= 0 || K % RQ_BLOCK_CODES != 0 || K > RQ_MAX_K || N <= 0 || N > (int64_t) 1 << 24) return RQ_E_UNSUPPORTED;
+    const PreparedLayout L = prepared_layout(K, N);
+    if (prepared_bytes < L.bytes || (reinterpret_cast<uintptr_t>(prepared_dev) & 255) != 0) return RQ_E_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(w_blocks_dev) & 15) != 0) return RQ_E_ARGUMENT;
+    return (int) launch_prepare(w_blocks_dev, L, reinterpret_cast<uint8_t *>(prepared_dev), (hipStream_t) stream);
+}
+
+size_t rq_w4a4_workspace_bytes(int type, int64_t K, int64_t N, int64_t M) {
+    if (!shape_ok(type, K, N, M)) return 0;
+    return workspace_layout(K, N, M < 1 ? 1 : M).bytes;
+}
+
+int rq_w4a4_mul_mat(int type, const void *prepared_dev, int64_t K, int64_t N, const float *x_dev, int64_t ldx,
+                    int64_t M, float *y_dev, int64_t ldy, float clip, int64_t n_rot, void *workspace_dev,
+                    size_t workspace_bytes, rq_stream_t stream) {
+    return run_products(type, 1, &prepared_dev, K, &N, x_dev, ldx, M, &y_dev, &ldy, clip, n_rot, workspace_dev,
+                        workspace_bytes, (hipStream_t) stream);
+}
+
+int rq_w4a4_mul_mat_fused(int type, int n, const void *const *prepared_dev, int64_t K, const int64_t *N,
+                          const float *x_dev, int64_t ldx, int64_t M, float *const *y_dev, const int64_t *ldy,
+                          float clip, int64_t n_rot, void *workspace_dev, size_t workspace_bytes,
+                          rq_stream_t stream) {
+    return run_products(type, n, prepared_dev, K, N, x_dev, ldx, M, y_dev, ldy, clip, n_rot, workspace_dev,
+                        workspace_bytes, (hipStream_t) stream);
+}
+
+int rq_w4a4_hadamard(const float *x_dev, int64_t ldx, int64_t M, int64_t K, int64_t n_rot, float *out_dev,
+                     int64_t ldo, rq_stream_t stream) {
+    if (!x_dev || !out_dev) return RQ_E_ARGUMENT;
+    if (K <= 0 || K % 4 != 0 || K > RQ_MAX_K || M < 0) return RQ_E_UNSUPPORTED;
+    if (ldx < K || ldo < K || (ldx * 4) % 16 != 0 || (ldo * 4) % 16 != 0) return RQ_E_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(x_dev) & 15) != 0 || (reinterpret_cast<uintptr_t>(out_dev) & 15) != 0) return RQ_E_ARGUMENT;
+    int p, m;
+    if (!rotation_of(RQ_TYPE_W4A4H, K, n_rot, p, m)) return RQ_E_ARGUMENT;
+    if (M == 0) return 0;
+    RotQuantArgs q;
+    memset(&q, 0, sizeof q);
+    q.x = x_dev;
+    q.ldx = ldx;
+    q.M = (int) M;
+    q.K = (int) K;
+    q.rotate = 1;
+    q.n_rot = (int) n_rot;
+    q.p = p;
+    q.m = m;
+    q.scale = 1.0f / sqrtf((float) n_rot);
+    q.clip = 1.0f;
+    q.mode = kActRotateOnly;
+    q.out_f32 = out_dev;
+    q.ldo = ldo;
+    return (int) launch_rotate_quant(q, (hipStream_t) stream);
+}
+
+int rq_w4a4_quantize_act(int type, const float *x_dev, int64_t ldx, int64_t M, int64_t K, float clip, int64_t n_rot,
+                         void *blocks_dev, rq_stream_t stream) {
+    if (!x_dev || !blocks_dev) return RQ_E_ARGUMENT;
+    if (type != RQ_TYPE_A4 && type != RQ_TYPE_A4H) return RQ_E_UNSUPPORTED;
+    if (K <= 0 || K % RQ_BLOCK_CODES != 0 || K > RQ_MAX_K || M < 0) return RQ_E_UNSUPPORTED;
+    if (env().act_group != 64) return RQ_E_UNSUPPORTED;
+    if (!(clip > 0.0f) || !isfinite(clip)) return RQ_E_ARGUMENT;
+    if (ldx < K || (ldx * 4) % 16 != 0 || (reinterpret_cast<uintptr_t>(x_dev) & 15) != 0) return RQ_E_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(blocks_dev) & 15) != 0) return RQ_E_ARGUMENT;
+    const bool had = type == RQ_TYPE_A4H;
+    int p, m;
+    if (!rotation_of(had ? RQ_TYPE_W4A4H : RQ_TYPE_W4A4, K, n_rot, p, m)) return RQ_E_ARGUMENT;
+    if (M == 0) return 0;
+    RotQuantArgs q;
+    memset(&q, 0, sizeof q);
+    q.x = x_dev;
+    q.ldx = ldx;
+    q.M = (int) M;
+    q.K = (int) K;
+    q.rotate = had;
+    q.n_rot = (int) (had ? n_rot : K);
+    q.p = p;
+    q.m = m;
+    q.scale = 1.0f / sqrtf((float) q.n_rot);
+    q.clip = clip;
+    q.mode = kActBlocks;
+    q.blocks = blocks_dev;
+    q.len_field = (int32_t) (had ? n_rot : K);
+    q.u = nullptr;  // the token unit goes into the block headers
+    return (int) launch_rotate_quant(q, (hipStream_t) stream);
+}
+
+}  // extern "C"

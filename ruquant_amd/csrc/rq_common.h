@@ -1,0 +1,166 @@
+// Shared definitions of the gfx950 W4A4 / W4A4H MUL_MAT library: memory layouts and launch-side helpers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/rq_w4a4.h"
+
+namespace rq {
+
+constexpr int kGroup      = 64;   // activation group: one zero point and one multiplier per 64 inputs
+constexpr int kPanelRows  = 64;   // weight rows per panel: one wavefront lane per row on the GEMV path
+constexpr int kTermShift  = 4;    // RQ_TERM_SHIFT (reference patch line 39)
+constexpr int kGemvTokens = 8;    // tokens per GEMV pass; the activation slot stride of the int4 layout
+constexpr int kGemmTokens = 128;  // token tile of the MFMA GEMM; int8 activations are padded to it
+
+// ---------------------------------------------------------------------------------------------------
+// Prepared weight (written once by rq_w4a4_prepare, read by every product kernel).
+//
+//   codes : n_panels x ng x 2 halves x 64 rows x 16 bytes. Row r of panel P, group g (inputs 64g..64g+63),
+//           half h (inputs 32h..32h+31 of the group) is the 16 bytes at
+//           (((P * ng + g) * 2 + h) * 64 + r) * 16: four code words in the tensor's own nibble order.
+//           A wavefront with lane = row reads one group of its 64 rows as two fully coalesced 1 KiB loads;
+//           an MFMA tile of 16 rows reads 256-byte runs.
+//   s_w   : n_panels x 64 floats (rows past N are zero).
+//   kmul  : n_panels x ng x 64 bytes, the integer weight multiplier of (row, group): 1 for legacy headers.
+//   flags : one int32; bit 0 set when any multiplier differs from 1 (kernels branch on it, uniformly).
+// ---------------------------------------------------------------------------------------------------
+struct PreparedLayout {
+    int64_t K, N;
+    int     ng;        // K / 64
+    int     n_panels;  // ceil(N / 64)
+    size_t  off_codes, off_sw, off_kmul, off_flags, bytes;
+};
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
+    PreparedLayout L;
+    L.K = K;
+    L.N = N;
+    L.ng = (int) (K / kGroup);
+    L.n_panels = (int) ((N + kPanelRows - 1) / kPanelRows);
+    size_t off = 0;
+    L.off_codes = off;
+    off = align_up(off + (size_t) L.n_panels * L.ng * 2048, 256);
+    L.off_sw = off;
+    off = align_up(off + (size_t) L.n_panels * kPanelRows * sizeof(float), 256);
+    L.off_kmul = off;
+    off = align_up(off + (size_t) L.n_panels * L.ng * kPanelRows, 256);
+    L.off_flags = off;
+    off = align_up(off + 256, 256);
+    L.bytes = off;
+    return L;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Workspace of one rq_w4a4_mul_mat call.
+//
+//   u      : Mp floats, the token units.
+//   act    : either the int4 form for the GEMV  ([chunk][g][8 token slots][8 words], codes q - 8, the
+//            tensor's nibble order) or the int8 form for the MFMA GEMM ([g][quarter][Mp][16 bytes], values q - z
+//            in the byte order the weight unpack produces).
+//   mz     : int4 form: [chunk][g][8] int32 = m | (8 - z) << 8 ... ; int8 form: [g][Mp] bytes = m.
+//   totals : split-K int32 sums [8 tokens][n_panels * 64] and one arrival counter per panel.
+// ---------------------------------------------------------------------------------------------------
+struct WorkspaceLayout {
+    int64_t Mp;       // tokens padded to the GEMM tile
+    int     chunks;   // ceil(M / 8)
+    size_t  off_u, off_act, off_mz, off_tot, off_cnt, bytes;
+    size_t  tot_ints, cnt_ints;
+};
+
+inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
+    WorkspaceLayout W;
+    const int ng = (int) (K / kGroup);
+    const int n_panels = (int) ((N + kPanelRows - 1) / kPanelRows);
+    W.Mp = (M + kGemmTokens - 1) / kGemmTokens * kGemmTokens;
+    W.chunks = (int) ((M + kGemvTokens - 1) / kGemvTokens);
+    size_t off = 0;
+    W.off_u = off;
+    off = align_up(off + (size_t) (W.Mp > (int64_t) W.chunks * 8 ? W.Mp : (int64_t) W.chunks * 8) * sizeof(float), 256);
+    const size_t act_q4 = (size_t) W.chunks * ng * kGemvTokens * 32;
+    const size_t act_i8 = (size_t) ng * W.Mp * 64;
+    W.off_act = off;
+    off = align_up(off + (act_q4 > act_i8 ? act_q4 : act_i8), 256);
+    const size_t mz_q4 = (size_t) W.chunks * ng * kGemvTokens * sizeof(int32_t);
+    const size_t mz_i8 = (size_t) ng * W.Mp;
+    W.off_mz = off;
+    off = align_up(off + (mz_q4 > mz_i8 ? mz_q4 : mz_i8), 256);
+    W.tot_ints = (size_t) kGemvTokens * n_panels * kPanelRows;
+    W.cnt_ints = (size_t) n_panels;
+    W.off_tot = off;
+    off = align_up(off + W.tot_ints * sizeof(int32_t), 256);
+    W.off_cnt = off;
+    off = align_up(off + W.cnt_ints * sizeof(int32_t), 256);
+    W.bytes = off;
+    return W;
+}
+
+// Output forms of the rotate + quantize kernel.
+enum ActMode : int {
+    kActRotateOnly = 0,  // fp32 rotated rows (rq_w4a4_hadamard)
+    kActBlocks     = 1,  // the reference's A4 / A4H block rows (rq_w4a4_quantize_act)
+    kActQ4         = 2,  // int4 codes + (m, 8 - z) words for the GEMV
+    kActI8         = 3,  // int8 (q - z) + m bytes for the MFMA GEMM
+};
+
+struct RotQuantArgs {
+    const float *x;      // M rows, stride ldx floats
+    int64_t      ldx;
+    int          M, K;
+    int          rotate; // 0: quantize x as is (W4A4); 1: rotate blocks of n_rot first (W4A4H)
+    int          n_rot, p, m;
+    float        scale;  // 1 / sqrtf(n_rot), computed on the host exactly as the reference does
+    float        clip;
+    int          mode;
+    // outputs
+    float       *out_f32;  int64_t ldo;   // kActRotateOnly
+    void        *blocks;                  // kActBlocks
+    int32_t      len_field;               // kActBlocks: pad[1] of the activation blocks (K or n_rot)
+    float       *u;
+    uint32_t    *act;                     // kActQ4 / kActI8
+    void        *mz;
+    int          Mp;                      // kActI8: padded token count (rows M..Mp-1 are zero filled)
+    // split-K scratch to clear (blocks past the token blocks do it)
+    int32_t     *zero_ptr;
+    int64_t      zero_ints;
+    int          token_blocks;            // number of leading blocks that process tokens
+};
+
+hipError_t launch_rotate_quant(const RotQuantArgs &a, hipStream_t stream);
+
+struct GemvArgs {
+    const uint8_t  *prepared;
+    PreparedLayout  L;
+    const uint32_t *act;    // int4 activation form of this chunk
+    const int32_t  *mz;
+    const float    *u;      // units of this chunk's tokens
+    float          *y;      // first token row of this chunk
+    int64_t         ldy;
+    int             T;      // 1..8 tokens
+    int32_t        *tot;    // split-K sums (zeroed)
+    int32_t        *cnt;    // arrival counters (zeroed)
+};
+hipError_t launch_gemv(const GemvArgs &a, hipStream_t stream);
+int gemv_ksplit(const PreparedLayout &L);
+
+struct GemmArgs {
+    const uint8_t  *prepared;
+    PreparedLayout  L;
+    const uint8_t  *act8;   // [g][quarter][Mp][16]
+    const uint8_t  *m8;     // [g][Mp]
+    const float    *u;      // [Mp]
+    float          *y;
+    int64_t         ldy;
+    int             M, Mp;
+};
+hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
+
+hipError_t launch_prepare(const void *blocks, const PreparedLayout &L, uint8_t *prepared, hipStream_t stream);
+
+bool hadamard_factor(int64_t n, int &p, int &m);
+
+}  // namespace rq

@@ -1,0 +1,336 @@
+// Online Hadamard (Paley x Sylvester) and per-token asymmetric int4 activation quantizer for gfx950.
+//
+// One workgroup owns one token: the whole row (up to 32768 floats) lives in the CU's 160 KiB LDS from the
+// global load to the last code word, so the rotated activations never travel through HBM.
+//
+// Bit-exactness with the CPU reference (ggml_rq_hadamard, reference patch lines 2450-2485, and
+// rq_quantize_row_a, lines 2639-2679) rests on three rules that this file keeps:
+//   * Sylvester stages are exact pairs (a + b, a - b), stride ascending; which lane computes a pair is free.
+//   * The Paley stage adds the p chunk values of a column strictly in ascending chunk order, starting from
+//     +0.0f, one rounding per add; the signs are compile-time constants so each term is one v_add / v_sub.
+//   * Every product, sum and quotient of the quantizer is a separate correctly rounded fp32 operation
+//     (no contraction, IEEE division, denormals kept).
+#include "rq_common.h"
+
+#pragma clang fp contract(off)
+
+namespace rq {
+
+namespace {
+
+constexpr int kNT = 512;  // threads per token workgroup
+
+// ---- Paley construction I, as signs: neg[i][a] is true where A[i][a] = -1 (reference lines 2433-2448) ----
+template <int P>
+struct PaleyTable {
+    bool neg[P][P];
+};
+
+template <int P>
+constexpr PaleyTable<P> make_paley() {
+    PaleyTable<P> t{};
+    constexpr int q = P - 1;
+    bool residue[P] = {};
+    for (int r = 1; r < q; ++r) residue[(r * r) % q] = true;
+    for (int i = 0; i < P; ++i) {
+        for (int a = 0; a < P; ++a) {
+            bool n = false;
+            if (i == a || i == 0) {
+                n = false;                       // diagonal and first row are +1
+            } else if (a == 0) {
+                n = true;                        // first column below the diagonal is -1
+            } else {
+                n = !residue[(((a - i) % q) + q) % q];
+            }
+            t.neg[i][a] = n;
+        }
+    }
+    return t;
+}
+
+// outputs 4S .. 4S+3 of one column: acc = ((0 +- c0) +- c1) ... in ascending chunk order
+template <int P, int S>
+__device__ __forceinline__ void paley_slice(const float (&col)[P], float (&out)[4]) {
+    constexpr PaleyTable<P> T = make_paley<P>();
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < P; ++i) {
+            acc = T.neg[i][4 * S + o] ? acc - col[i] : acc + col[i];
+        }
+        out[o] = acc;
+    }
+}
+
+template <int P, int S = 0>
+__device__ __forceinline__ void paley_pick(int s, const float (&col)[P], float (&out)[4]) {
+    if (s == S) {
+        paley_slice<P, S>(col, out);
+    } else if constexpr (S + 1 < P / 4) {
+        paley_pick<P, S + 1>(s, col, out);
+    }
+}
+
+// all P outputs of one column, written back in place (the column is private to the calling thread)
+template <int P, int S = 0>
+__device__ __forceinline__ void paley_column(const float (&col)[P], float *dst, int stride, float scale) {
+    float out[4];
+    paley_slice<P, S>(col, out);
+#pragma unroll
+    for (int o = 0; o < 4; ++o) dst[(4 * S + o) * stride] = out[o] * scale;
+    if constexpr (S + 1 < P / 4) paley_column<P, S + 1>(col, dst, stride, scale);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+template <int P, bool SLICED>
+__global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs a) {
+    extern __shared__ __align__(16) float smem[];
+    __shared__ float s_red[kNT / 64];
+
+    const int tid = threadIdx.x;
+    if ((int) blockIdx.x >= a.token_blocks) {
+        // blocks past the tokens clear the split-K sums and arrival counters of the product kernel
+        const int64_t i0 = ((int64_t) (blockIdx.x - a.token_blocks) * kNT + tid) * 4;
+        if (i0 + 3 < a.zero_ints) {
+            *reinterpret_cast<int4 *>(a.zero_ptr + i0) = make_int4(0, 0, 0, 0);
+        } else {
+            for (int64_t i = i0; i < a.zero_ints; ++i) a.zero_ptr[i] = 0;
+        }
+        return;
+    }
+
+    const int t = blockIdx.x;
+    const int K = a.K;
+    const int ng = K / kGroup;
+    float *buf = smem;
+    float *alt = smem + K;                       // second row buffer (SLICED only)
+    float *g_lo = smem + (SLICED ? 2 * K : K);
+    float *g_hi = g_lo + ng;
+
+    const float *xr = a.x + (int64_t) t * a.ldx;
+    for (int i = tid * 4; i < K; i += kNT * 4) {
+        *reinterpret_cast<float4 *>(buf + i) = *reinterpret_cast<const float4 *>(xr + i);
+    }
+    __syncthreads();
+
+    if (a.rotate) {
+        const int m = a.m;
+        // Sylvester butterflies inside every chunk of m, stride 1, 2, 4, ... (reference lines 2454-2464)
+        if (m > 1) {
+            const int half = m >> 1;
+            const int lhalf = __ffs(half) - 1;
+            for (int h = 1; h < m; h <<= 1) {
+                for (int q = tid; q < (K >> 1); q += kNT) {
+                    const int c = q >> lhalf, r = q & (half - 1);
+                    const int j = ((r & ~(h - 1)) << 1) | (r & (h - 1));
+                    float *v = buf + c * m + j;
+                    const float lo = v[0], up = v[h];
+                    v[0] = lo + up;
+                    v[h] = lo - up;
+                }
+                __syncthreads();
+            }
+        }
+        if constexpr (P > 1) {
+            // Paley across the P chunks of every rotation block (reference lines 2466-2482), then the scale
+            const int ncols = K / P;  // columns of all rotation blocks of this token
+            if constexpr (SLICED) {
+                for (int id = tid; id < (K >> 2); id += kNT) {
+                    const int s = id / ncols, cidx = id - s * ncols;
+                    const int rb = cidx / m, j = cidx - rb * m;
+                    const float *src = buf + rb * a.n_rot + j;
+                    float col[P];
+#pragma unroll
+                    for (int i = 0; i < P; ++i) col[i] = src[i * m];
+                    float out[4];
+                    paley_pick<P>(s, col, out);
+                    float *dst = alt + rb * a.n_rot + j + 4 * s * m;
+#pragma unroll
+                    for (int o = 0; o < 4; ++o) dst[o * m] = out[o] * a.scale;
+                }
+                __syncthreads();
+                float *tmp = buf; buf = alt; alt = tmp;
+            } else {
+                for (int cidx = tid; cidx < ncols; cidx += kNT) {
+                    const int rb = cidx / m, j = cidx - rb * m;
+                    float *src = buf + rb * a.n_rot + j;
+                    float col[P];
+#pragma unroll
+                    for (int i = 0; i < P; ++i) col[i] = src[i * m];
+                    paley_column<P>(col, src, m, a.scale);
+                }
+                __syncthreads();
+            }
+        } else {
+            for (int i = tid; i < K; i += kNT) buf[i] = buf[i] * a.scale;
+            __syncthreads();
+        }
+    }
+
+    if (a.mode == kActRotateOnly) {
+        float *o = a.out_f32 + (int64_t) t * a.ldo;
+        for (int i = tid * 4; i < K; i += kNT * 4) {
+            *reinterpret_cast<float4 *>(o + i) = *reinterpret_cast<const float4 *>(buf + i);
+        }
+        return;
+    }
+
+    // ---- group ranges [min(x,0), max(x,0)] * clip and the token's widest range (reference lines 2646-2654)
+    const int nw = K >> 3;  // code words of this token: a thread per word, 8 lanes per group of 64
+    float rmax = 0.0f;
+    for (int w0 = 0; w0 < nw; w0 += kNT) {
+        const int w = w0 + tid;
+        const bool on = w < nw;
+        float mn = 0.0f, mx = 0.0f;
+        if (on) {
+            const float4 v0 = *reinterpret_cast<const float4 *>(buf + 8 * w);
+            const float4 v1 = *reinterpret_cast<const float4 *>(buf + 8 * w + 4);
+            mn = fminf(fminf(fminf(fminf(mn, v0.x), fminf(v0.y, v0.z)), fminf(fminf(v0.w, v1.x), fminf(v1.y, v1.z))), v1.w);
+            mx = fmaxf(fmaxf(fmaxf(fmaxf(mx, v0.x), fmaxf(v0.y, v0.z)), fmaxf(fmaxf(v0.w, v1.x), fmaxf(v1.y, v1.z))), v1.w);
+        }
+#pragma unroll
+        for (int off = 1; off < 8; off <<= 1) {
+            mn = fminf(mn, __shfl_xor(mn, off, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        }
+        const float lo = mn * a.clip, hi = mx * a.clip;
+        if (on) {
+            if ((tid & 7) == 0) {
+                g_lo[w >> 3] = lo;
+                g_hi[w >> 3] = hi;
+            }
+            rmax = fmaxf(rmax, hi - lo);
+        }
+    }
+    rmax = wave_max(rmax);
+    if ((tid & 63) == 0) s_red[tid >> 6] = rmax;
+    __syncthreads();
+    float R = s_red[0];
+#pragma unroll
+    for (int i = 1; i < kNT / 64; ++i) R = fmaxf(R, s_red[i]);
+    if (R == 0.0f) R = 2.0f;
+    const float u = R / 3825.0f;  // 15 * 255
+    if (tid == 0 && a.u != nullptr) a.u[t] = u;
+
+    // ---- per group multiplier and zero point, per value code (reference lines 2662-2677)
+    for (int w0 = 0; w0 < nw; w0 += kNT) {
+        const int w = w0 + tid;
+        const bool on = w < nw;
+        const int wc = on ? w : 0;
+        const int g = wc >> 3;
+        const float lo = g_lo[g], hi = g_hi[g];
+        const int mg = (int) fminf(fmaxf(ceilf(((hi - lo) * 255.0f) / R), 1.0f), 255.0f);
+        const float inv = 1.0f / ((float) mg * u);
+        const float zf = fminf(fmaxf(rintf(-lo * inv), 0.0f), 15.0f);
+        const int z = (int) zf;
+        const float4 v0 = *reinterpret_cast<const float4 *>(buf + 8 * wc);
+        const float4 v1 = *reinterpret_cast<const float4 *>(buf + 8 * wc + 4);
+        const float f[8] = { v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w };
+        int q[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) q[j] = (int) fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
+
+        if (a.mode == kActI8) {
+            // bytes q - z in the order the weight unpack yields: even codes of the word, then odd codes
+            uint32_t lo4 = 0, hi4 = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                lo4 |= (uint32_t) ((q[2 * j] - z) & 0xFF) << (8 * j);
+                hi4 |= (uint32_t) ((q[2 * j + 1] - z) & 0xFF) << (8 * j);
+            }
+            if (on) {
+                // [group][quarter of the group][token][16 bytes]: a token tile of one quarter is contiguous
+                uint32_t *dst = a.act + (((size_t) g * 4 + ((w & 7) >> 1)) * a.Mp + t) * 4 + (w & 1) * 2;
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(lo4, hi4);
+                if ((tid & 7) == 0) reinterpret_cast<uint8_t *>(a.mz)[(size_t) g * a.Mp + t] = (uint8_t) mg;
+            }
+            continue;
+        }
+
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) word |= (uint32_t) ((q[j] - 8) & 0xF) << (4 * j);
+
+        if (a.mode == kActQ4) {
+            if (on) {
+                const int chunk = t >> 3, slot = t & 7;
+                const size_t cell = ((size_t) chunk * ng + g) * kGemvTokens + slot;
+                a.act[cell * 8 + (w & 7)] = word;
+                if ((tid & 7) == 0) reinterpret_cast<int32_t *>(a.mz)[cell] = mg | ((8 - z) & 0xFF) << 8;
+            }
+        } else {  // kActBlocks: the reference's A4 / A4H storage (reference lines 2656-2661, 2667-2669)
+            const int base = tid & 32;  // lanes base, base+8, base+16, base+24 hold the block's four groups
+            uint32_t zs = 0, ms = 0;
+#pragma unroll
+            for (int sg = 0; sg < 4; ++sg) {
+                zs |= (uint32_t) __shfl(z, base + 8 * sg, 64) << (4 * sg);
+                ms |= (uint32_t) __shfl(mg, base + 8 * sg, 64) << (8 * sg);
+            }
+            if (on) {
+                rq_block_w4a4 *blk = reinterpret_cast<rq_block_w4a4 *>(a.blocks) + (size_t) t * (K / RQ_BLOCK_CODES) + (w >> 5);
+                blk->qs[w & 31] = word;
+                if ((w & 31) == 0) {
+                    blk->d = u;
+                    blk->sum = (int32_t) ((2u << 16) | zs);
+                    blk->pad[0] = (int32_t) ms;
+                    blk->pad[1] = a.len_field;
+                }
+            }
+        }
+    }
+}
+
+template <int P, bool SLICED>
+hipError_t launch_one(const RotQuantArgs &a, size_t lds, int grid, hipStream_t stream) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_rotate_quant_kernel<P, SLICED>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((rq_rotate_quant_kernel<P, SLICED>), dim3(grid), dim3(kNT), lds, stream, a);
+    return hipGetLastError();
+}
+
+template <int P>
+hipError_t launch_p(const RotQuantArgs &a, int grid, hipStream_t stream) {
+    const size_t stats = (size_t) 2 * (a.K / kGroup) * sizeof(float);
+    const size_t lds_sliced = (size_t) 2 * a.K * sizeof(float) + stats;
+    if (P > 1 && lds_sliced <= 160 * 1024 - 64) {
+        return launch_one<P, (P > 1)>(a, lds_sliced, grid, stream);
+    }
+    return launch_one<P, false>(a, (size_t) a.K * sizeof(float) + stats, grid, stream);
+}
+
+}  // namespace
+
+hipError_t launch_rotate_quant(const RotQuantArgs &a, hipStream_t stream) {
+    const int zero_blocks = (int) ((a.zero_ints + (int64_t) kNT * 4 - 1) / ((int64_t) kNT * 4));
+    RotQuantArgs b = a;
+    b.token_blocks = a.M;
+    const int grid = a.M + zero_blocks;
+    if (grid == 0) return hipSuccess;
+    const int p = a.rotate ? a.p : 1;
+    switch (p) {
+        case 1:   return launch_p<1>(b, grid, stream);
+        case 12:  return launch_p<12>(b, grid, stream);
+        case 20:  return launch_p<20>(b, grid, stream);
+        case 44:  return launch_p<44>(b, grid, stream);
+        case 60:  return launch_p<60>(b, grid, stream);
+        case 68:  return launch_p<68>(b, grid, stream);
+        case 72:  return launch_p<72>(b, grid, stream);
+        case 84:  return launch_p<84>(b, grid, stream);
+        case 104: return launch_p<104>(b, grid, stream);
+        case 108: return launch_p<108>(b, grid, stream);
+        default:  return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace rq

@@ -1,0 +1,70 @@
+"""Loads librq_w4a4.so and declares the prototypes of include/rq_w4a4.h."""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "librq_w4a4.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def build_library(jobs=8):
+    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU)."""
+    subprocess.run(["make", "-C", CSRC, "-B", "-j%d" % jobs], check=True)
+    return LIB_PATH
+
+
+_lib = None
+
+c_f32p = ctypes.POINTER(ctypes.c_float)
+c_i64p = ctypes.POINTER(ctypes.c_int64)
+c_intp = ctypes.POINTER(ctypes.c_int)
+
+PROTOTYPES = {
+    "rq_w4a4_abi_version": (ctypes.c_int, []),
+    "rq_w4a4_supported": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                         ctypes.c_int64, ctypes.c_int64]),
+    "rq_w4a4_hadamard_factor": (ctypes.c_int, [ctypes.c_int64, c_intp, c_intp]),
+    "rq_w4a4_resolve_clip": (ctypes.c_float, [ctypes.c_void_p, ctypes.c_int]),
+    "rq_w4a4_tensor_rot": (ctypes.c_int64, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64]),
+    "rq_w4a4_act_group": (ctypes.c_int, []),
+    "rq_w4a4_prepared_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64]),
+    "rq_w4a4_prepare": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
+                                       ctypes.c_size_t, ctypes.c_void_p]),
+    "rq_w4a4_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64]),
+    "rq_w4a4_mul_mat": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                       ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
+                                       ctypes.c_int64, ctypes.c_float, ctypes.c_int64, ctypes.c_void_p,
+                                       ctypes.c_size_t, ctypes.c_void_p]),
+    "rq_w4a4_mul_mat_fused": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_void_p),
+                                             ctypes.c_int64, c_i64p, ctypes.c_void_p, ctypes.c_int64,
+                                             ctypes.c_int64, ctypes.POINTER(ctypes.c_void_p), c_i64p,
+                                             ctypes.c_float, ctypes.c_int64, ctypes.c_void_p, ctypes.c_size_t,
+                                             ctypes.c_void_p]),
+    "rq_w4a4_hadamard": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                        ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
+    "rq_w4a4_quantize_act": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                            ctypes.c_int64, ctypes.c_float, ctypes.c_int64, ctypes.c_void_p,
+                                            ctypes.c_void_p]),
+}
+
+
+def load_library():
+    """Returns the ctypes handle of librq_w4a4.so; raises LibraryMissing when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise LibraryMissing(
+                "%s is missing: build it with `make -C %s` (or __graft_entry__.build()); there is no fallback path"
+                % (LIB_PATH, CSRC))
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib

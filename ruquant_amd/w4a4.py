@@ -1,0 +1,160 @@
+"""Host-side mirror of the reference's W4A4 operator interface over the C ABI.
+
+Names follow the reference's backend entry points (patches/llama.cpp-ruquant.patch, rq-w4a4.cuh, lines
+2391-2401 of the patch): ``supported`` <-> ggml_cuda_rq_w4a4_supported, ``W4A4Weight.ready`` <->
+ggml_cuda_rq_w4a4_ready, ``mul_mat`` <-> ggml_cuda_mul_mat_rq_w4a4, ``mul_mat_fused`` <->
+ggml_cuda_mul_mat_rq_w4a4_fused. A ``W4A4Weight`` plays the part of the ggml weight tensor plus the
+``rq_tensor_info`` the reference hangs on ``src0->extra`` at first use (patch lines 2027-2043).
+
+torch owns device memory and the stream; every computation happens inside librq_w4a4.so.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from .lib import load_library
+
+TYPE_W4A4, TYPE_W4A4H, TYPE_A4, TYPE_A4H = 44, 45, 46, 47
+BLOCK_DTYPE = np.dtype([("d", "<f4"), ("sum", "<i4"), ("pad", "<i4", (2,)), ("qs", "<u4", (32,))])
+
+
+class RqError(RuntimeError):
+    pass
+
+
+_ERRORS = {-1: "unsupported shape or type", -2: "workspace / prepared buffer too small or misaligned",
+           -3: "bad argument"}
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise RqError("%s failed: %s" % (what, _ERRORS.get(rc, "hipError_t %d" % rc)))
+
+
+def _stream_ptr():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _device_bytes(n, device):
+    # torch's caching allocator returns 512-byte aligned blocks; the ABI needs 256
+    t = torch.empty(max(int(n), 256), dtype=torch.uint8, device=device)
+    assert t.data_ptr() % 256 == 0
+    return t
+
+
+def hadamard_factor(n):
+    p, m = ctypes.c_int(0), ctypes.c_int(0)
+    ok = load_library().rq_w4a4_hadamard_factor(int(n), ctypes.byref(p), ctypes.byref(m))
+    return (p.value, m.value) if ok else None
+
+
+def supported(type_, K, N, M, ldx_bytes=None, ldy_bytes=None):
+    ldx_bytes = 4 * K if ldx_bytes is None else ldx_bytes
+    ldy_bytes = 4 * N if ldy_bytes is None else ldy_bytes
+    return bool(load_library().rq_w4a4_supported(type_, K, N, M, ldx_bytes, ldy_bytes))
+
+
+def resolve_clip(block0, type_):
+    """block0: the first block of the tensor (numpy, host). Environment > header pad[1] > 1."""
+    b = np.ascontiguousarray(block0).view(np.uint8)
+    return float(load_library().rq_w4a4_resolve_clip(b.ctypes.data, type_))
+
+
+def tensor_rot(block0, type_, K):
+    b = np.ascontiguousarray(block0).view(np.uint8)
+    return int(load_library().rq_w4a4_tensor_rot(b.ctypes.data, type_, K))
+
+
+class W4A4Weight:
+    """A W4A4 / W4A4H weight tensor on the GPU: [N, K/256] blocks as ggml stores them, plus what the first use
+    derives (clip, Hadamard length, the prepared streaming form)."""
+
+    def __init__(self, blocks, type_, device="cuda:0", keep_blocks=True):
+        blocks = np.ascontiguousarray(blocks)
+        assert blocks.dtype == BLOCK_DTYPE and blocks.ndim == 2
+        self.type = int(type_)
+        self.N, nb = blocks.shape
+        self.K = nb * 256
+        self.device = torch.device(device)
+        L = load_library()
+        # first use: header of block 0 (the reference reads it back from the device, patch lines 2030-2040)
+        self.clip = resolve_clip(blocks[0, 0], self.type)
+        self.n_rot = tensor_rot(blocks[0, 0], self.type, self.K)
+        if self.type == TYPE_W4A4H and self.n_rot < 0:
+            raise RqError("W4A4H: Hadamard length %d does not divide this row of %d"
+                          % (int(blocks[0, 0]["pad"][0]), self.K))
+        raw = torch.from_numpy(blocks.view(np.uint8).reshape(-1).copy()).to(self.device)
+        nbytes = L.rq_w4a4_prepared_bytes(self.K, self.N)
+        if nbytes == 0:
+            raise RqError("unsupported weight shape K=%d N=%d" % (self.K, self.N))
+        self.prepared = _device_bytes(nbytes, self.device)
+        with torch.cuda.device(self.device):
+            _check(L.rq_w4a4_prepare(raw.data_ptr(), self.K, self.N, self.prepared.data_ptr(), nbytes,
+                                     _stream_ptr()), "rq_w4a4_prepare")
+        self.blocks = raw if keep_blocks else None
+        self.ready = True
+
+    def workspace(self, M):
+        n = load_library().rq_w4a4_workspace_bytes(self.type, self.K, self.N, M)
+        return _device_bytes(n, self.device)
+
+
+def mul_mat(weight, x, out=None, workspace=None, clip=None):
+    """y[M, N] = x[M, K] . W^T, bit-identical to the ggml-cpu W4A4 / W4A4H MUL_MAT."""
+    return mul_mat_fused([weight], x, outs=None if out is None else [out], workspace=workspace, clip=clip)[0]
+
+
+def mul_mat_fused(weights, x, outs=None, workspace=None, clip=None):
+    """Up to three weights of one type, K, clip and rotation length against the same activations."""
+    L = load_library()
+    w0 = weights[0]
+    assert x.is_cuda and x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1
+    M, K = x.shape
+    assert K == w0.K
+    for w in weights[1:]:
+        if (w.type, w.K, w.clip, w.n_rot) != (w0.type, w0.K, w0.clip, w0.n_rot):
+            raise RqError("weights cannot be fused: type, K, clip and rotation length must match")
+    if outs is None:
+        outs = [torch.empty((M, w.N), dtype=torch.float32, device=x.device) for w in weights]
+    n = len(weights)
+    Nmax = max(w.N for w in weights)
+    if workspace is None:
+        workspace = _device_bytes(L.rq_w4a4_workspace_bytes(w0.type, K, Nmax, M), x.device)
+    prepared = (ctypes.c_void_p * n)(*[w.prepared.data_ptr() for w in weights])
+    ys = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
+    Ns = (ctypes.c_int64 * n)(*[w.N for w in weights])
+    ldys = (ctypes.c_int64 * n)(*[o.stride(0) if o.shape[0] > 1 else o.shape[1] for o in outs])
+    ldx = x.stride(0) if M > 1 else K
+    with torch.cuda.device(x.device):
+        rc = L.rq_w4a4_mul_mat_fused(w0.type, n, prepared, K, Ns, x.data_ptr(), ldx, M, ys, ldys,
+                                     w0.clip if clip is None else clip, max(w0.n_rot, 0),
+                                     workspace.data_ptr(), workspace.numel(), _stream_ptr())
+    _check(rc, "rq_w4a4_mul_mat")
+    return outs
+
+
+def hadamard(x, n_rot=None):
+    """x[M, K] -> x diag(H, H, ...) with H of length n_rot (default K), as ggml_rq_hadamard does per block."""
+    L = load_library()
+    assert x.is_cuda and x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1
+    M, K = x.shape
+    out = torch.empty((M, K), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = L.rq_w4a4_hadamard(x.data_ptr(), x.stride(0) if M > 1 else K, M, K, n_rot or K, out.data_ptr(), K,
+                                _stream_ptr())
+    _check(rc, "rq_w4a4_hadamard")
+    return out
+
+
+def quantize_act(x, clip, hadamard_=False, n_rot=None):
+    """x[M, K] -> [M, K/256] activation blocks in the reference's A4 / A4H layout (numpy, host)."""
+    L = load_library()
+    assert x.is_cuda and x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1
+    M, K = x.shape
+    out = torch.zeros(M * (K // 256) * 144, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = L.rq_w4a4_quantize_act(TYPE_A4H if hadamard_ else TYPE_A4, x.data_ptr(), x.stride(0) if M > 1 else K,
+                                    M, K, clip, (n_rot or K) if hadamard_ else 0, out.data_ptr(), _stream_ptr())
+    _check(rc, "rq_w4a4_quantize_act")
+    return out.cpu().numpy().view(BLOCK_DTYPE).reshape(M, K // 256)

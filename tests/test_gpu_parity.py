@@ -1,0 +1,283 @@
+"""GPU parity: every stage of the HIP path against the CPU oracle, zero tolerance (bit patterns compared)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import ruquant_amd as rq
+from ruquant_amd import synth
+from tests.gpu_util import bits_equal, first_mismatch, adversarial_weights, adversarial_activations, run_gpu
+from tests.lcg import act_row, weight_row, fnv64
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "reference_known_answers.json")) as f:
+    KA = json.load(f)
+
+DEV = "cuda:0"
+
+
+def f32bits(x):
+    return "%08x" % int(np.asarray(x, dtype=np.float32).view(np.uint32))
+
+
+# ---------------------------------------------------------------- Hadamard (kernel 1)
+
+@pytest.mark.parametrize("case", KA["hadamard"], ids=lambda c: "k%d" % c["k"])
+def test_hadamard_reference_known_answers(case):
+    """The compiled reference's own outputs, no oracle involved."""
+    k = case["k"]
+    x = torch.from_numpy(act_row(k)[None, :]).to(DEV)
+    y = rq.hadamard(x).cpu().numpy()[0]
+    assert f32bits(y[0]) == case["h0"] and f32bits(y[1]) == case["h1"] and f32bits(y[-1]) == case["hlast"]
+    assert fnv64(y.astype("<f4").tobytes()) == case["fnv64"]
+
+
+@pytest.mark.parametrize("K,n_rot", [(256, 256), (256, 128), (256, 32), (768, 12), (1536, 1536), (1536, 768),
+                                       (4096, 4096), (5120, 5120), (5120, 2560), (6144, 6144), (17408, 17408),
+                                       (17408, 4352), (8192, 8192), (32768, 32768), (24576, 24576), (11264, 11264),
+                                       (15360, 15360), (18432, 18432), (21504, 21504), (26624, 26624), (27648, 27648),
+                                       (20480, 5120), (22528, 22528), (30720, 30720), (21760, 4352), (23040, 4608)])
+def test_hadamard_vs_oracle(oracle, K, n_rot):
+    rng = np.random.default_rng(K + n_rot)
+    M = 3
+    x = (rng.standard_normal((M, K)) * np.exp2(rng.integers(-6, 7, size=(M, K)))).astype(np.float32)
+    got = rq.hadamard(torch.from_numpy(x).to(DEV), n_rot).cpu().numpy()
+    want = np.stack([np.concatenate([oracle.hadamard(x[t, o:o + n_rot]) for o in range(0, K, n_rot)]) for t in range(M)])
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+def test_hadamard_signed_zero_and_strided_rows(oracle):
+    K = 1536
+    x = np.zeros((2, K + 64), dtype=np.float32)
+    x[0, :K] = -0.0
+    x[1, :K] = np.random.default_rng(0).standard_normal(K).astype(np.float32)
+    xd = torch.from_numpy(x).to(DEV)[:, :K]            # row stride K + 64 floats
+    got = rq.hadamard(xd).cpu().numpy()
+    want = np.stack([oracle.hadamard(x[t, :K]) for t in range(2)])
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+# ---------------------------------------------------------------- quantizer (kernel 2)
+
+@pytest.mark.parametrize("case", KA["quant"], ids=lambda c: "k%d_%s_%s" % (c["k"], "QH" if c["hadamard"] else "Q", c["clip"]))
+def test_quantizer_reference_known_answers(case):
+    k = case["k"]
+    clip = float(np.float32(float(case["clip"])))
+    x = torch.from_numpy(act_row(k)[None, :]).to(DEV)
+    a = rq.quantize_act(x, clip, hadamard_=case["hadamard"])[0]
+    assert f32bits(a["d"][0]) == case["u"]
+    assert "%08x" % (int(a["sum"][0]) & 0xFFFFFFFF) == case["sum0"]
+    assert "%08x" % (int(a["pad"][0, 0]) & 0xFFFFFFFF) == case["pad0"]
+    assert fnv64(a.tobytes()) == case["fnv64"]
+
+
+@pytest.mark.parametrize("K", [256, 1536, 5120, 17408, 32768])
+@pytest.mark.parametrize("had", [False, True])
+def test_quantizer_blocks_vs_oracle(oracle, K, had):
+    rng = np.random.default_rng(K)
+    M = 5
+    x = (rng.standard_normal((M, K)) * np.exp2((np.arange(K) // 64 % 7 - 3))).astype(np.float32)
+    x[1] = 0.0                                   # all-zero token: R = 2
+    x[2] = np.abs(x[2])                          # non-negative token: every zero point 0
+    x[3, ::2] = 0.0
+    clip = float(np.float32(0.9))
+    got = rq.quantize_act(torch.from_numpy(x).to(DEV), clip, hadamard_=had)
+    for t in range(M):
+        want = oracle.quantize_row_a4h(x[t], clip, K) if had else oracle.quantize_row_a(x[t], clip)
+        assert got[t].tobytes() == want.tobytes(), "token %d" % t
+
+
+# ---------------------------------------------------------------- MUL_MAT, the reference's test shapes
+
+def _shapes_reference():
+    shapes = []
+    for m in [1, 3, 8, 17, 64, 200]:
+        for k in [256, 512, 1536, 5120, 6144]:
+            shapes.append((136, m, k))
+    shapes.append((5120, 32, 17408))
+    for m in [1, 2, 4, 5, 8, 16, 24, 32, 48, 64, 65, 130]:
+        for k in [256, 6144]:
+            shapes.append((256, m, k))
+    shapes += [(192, 8, 5120), (1024, 8, 5120), (5120, 8, 17408)]
+    return shapes
+
+
+_WCACHE = {}
+
+
+def _weights(oracle, N, K, type_, wgroup=0):
+    key = (N, K, type_, wgroup)
+    if key not in _WCACHE:
+        blocks, wf = adversarial_weights(oracle, N, K, type_, wgroup=wgroup)
+        _WCACHE.clear()            # one at a time: the big ones are tens of MB
+        _WCACHE[key] = (blocks, wf, rq.W4A4Weight(blocks, type_, DEV))
+    return _WCACHE[key]
+
+
+@pytest.mark.parametrize("type_", [rq.TYPE_W4A4, rq.TYPE_W4A4H], ids=["w4a4", "w4a4h"])
+@pytest.mark.parametrize("N,M,K", sorted(_shapes_reference(), key=lambda s: (s[0], s[2], s[1])),
+                         ids=lambda v: str(v))
+def test_mul_mat_reference_shapes(oracle, type_, N, M, K):
+    blocks, wf, W = _weights(oracle, N, K, type_)
+    x = adversarial_activations(M, K, type_, wf)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=max(W.n_rot, 0))
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+@pytest.mark.parametrize("wgroup", [256, 64])
+@pytest.mark.parametrize("M", [3, 40])
+def test_mul_mat_weight_multipliers(oracle, wgroup, M):
+    """Headers that carry integer weight multipliers per block or per 64 inputs (patch lines 40-43)."""
+    N, K, type_ = 200, 1536, rq.TYPE_W4A4H
+    blocks, wf = adversarial_weights(oracle, N, K, type_, wgroup=wgroup)
+    assert ((blocks["sum"].view(np.uint32) >> 30) == 1).all()
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    x = adversarial_activations(M, K, type_, wf)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=K)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+def test_mul_mat_block_diagonal_rotation(oracle):
+    """Hadamard length shorter than the row (pad[0] = K / 4), as ruquant convert --rot-blocks writes."""
+    N, K, M, type_ = 128, 6144, 9, rq.TYPE_W4A4H
+    blocks, wf = adversarial_weights(oracle, N, K, type_, n_rot=K // 4)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    assert W.n_rot == K // 4
+    x = adversarial_activations(M, K, type_, wf)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=K // 4)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+def test_mul_mat_strided_input_and_output(oracle):
+    N, K, M, type_ = 320, 1536, 6, rq.TYPE_W4A4
+    blocks, wf = adversarial_weights(oracle, N, K, type_)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    x = adversarial_activations(M, K, type_, wf)
+    xd = torch.zeros((M, K + 128), dtype=torch.float32, device=DEV)
+    xd[:, :K] = torch.from_numpy(x).to(DEV)
+    out = torch.full((M, N + 32), -7.0, dtype=torch.float32, device=DEV)
+    rq.mul_mat(W, xd[:, :K], out=out[:, :N])
+    torch.cuda.synchronize()
+    want = oracle.mul_mat(type_, blocks, x, W.clip)
+    got = out.cpu().numpy()
+    assert bits_equal(got[:, :N], want), first_mismatch(got[:, :N], want)
+    assert (got[:, N:] == -7.0).all()
+
+
+def test_fused_matches_separate(oracle):
+    K, M, type_ = 5120, 4, rq.TYPE_W4A4H
+    ws, bl = [], []
+    for i, N in enumerate([384, 64, 1024]):
+        b = synth.random_weight_blocks(N, K, 10 + i, type_, clip=0.9)
+        bl.append(b)
+        ws.append(rq.W4A4Weight(b, type_, DEV))
+    x = synth.activations("outlier_channels", M, K, 5)
+    xd = torch.from_numpy(x).to(DEV)
+    outs = rq.mul_mat_fused(ws, xd)
+    torch.cuda.synchronize()
+    for b, w, o in zip(bl, ws, outs):
+        want = oracle.mul_mat(type_, b, x, w.clip, n_rot=K)
+        assert bits_equal(o.cpu().numpy(), want), first_mismatch(o.cpu().numpy(), want)
+
+
+# ---------------------------------------------------------------- the five benchmark configurations
+
+def test_config1_w4a4_k4096_n1024_m1(oracle):
+    K, N, M = 4096, 1024, 1
+    blocks = synth.random_weight_blocks(N, K, 0, rq.TYPE_W4A4)
+    W = rq.W4A4Weight(blocks, rq.TYPE_W4A4, DEV)
+    assert W.clip == 1.0
+    x = synth.activations("normal", M, K, 0)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(rq.TYPE_W4A4, blocks, x, 1.0)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 8])
+def test_config2_decode_gemv(oracle, M):
+    K, N = 5120, 5120
+    blocks = synth.random_weight_blocks(N, K, 2, rq.TYPE_W4A4H, clip=0.9)
+    W = rq.W4A4Weight(blocks, rq.TYPE_W4A4H, DEV)
+    assert W.clip == float(np.float32(0.9)) and W.n_rot == K
+    x = synth.activations("outlier_channels", M, K, 2)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(rq.TYPE_W4A4H, blocks, x, W.clip, n_rot=K)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+@pytest.mark.parametrize("M", [64, 512, 2048])
+def test_config3_prefill_gemm(oracle, M):
+    K, N = 5120, 17408
+    blocks = synth.random_weight_blocks(N, K, 3, rq.TYPE_W4A4H)
+    W = rq.W4A4Weight(blocks, rq.TYPE_W4A4H, DEV)
+    clip = float(np.float32(0.85))                # RQ_ACT_CLIP_H=0.85 in the reference's run; passed explicitly
+    x = synth.activations("student_t4", M, K, 3)
+    y = rq.mul_mat(W, torch.from_numpy(x).to(DEV), clip=clip)
+    torch.cuda.synchronize()
+    got = y.cpu().numpy()
+    want = oracle.mul_mat(rq.TYPE_W4A4H, blocks, x, clip, n_rot=K)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+@pytest.mark.parametrize("M", [1, 16, 2048])
+def test_config4_down_projection(oracle, M):
+    K, N = 17408, 5120
+    blocks = synth.random_weight_blocks(N, K, 4, rq.TYPE_W4A4H)
+    W = rq.W4A4Weight(blocks, rq.TYPE_W4A4H, DEV)
+    x = synth.activations("relu2", M, K, 4)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(rq.TYPE_W4A4H, blocks, x, 1.0, n_rot=K)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+def test_config5_transformer_layer_chain(oracle):
+    """Seven matmuls at M = 16 chained along the layer's dataflow: q, k, v <- x0; o <- q; gate, up <- o; down <- up."""
+    M, type_ = 16, rq.TYPE_W4A4H
+    shapes = dict(q=(5120, 6144), k=(5120, 1024), v=(5120, 1024), o=(6144, 5120), gate=(5120, 17408),
+                  up=(5120, 17408), down=(17408, 5120))
+    blocks = {n: synth.random_weight_blocks(No, Ki, 100 + i, type_) for i, (n, (Ki, No)) in enumerate(shapes.items())}
+    W = {n: rq.W4A4Weight(b, type_, DEV) for n, b in blocks.items()}
+    x0 = synth.activations("normal", M, 5120, 1)
+    xd = torch.from_numpy(x0).to(DEV)
+    q, k, v = rq.mul_mat_fused([W["q"], W["k"], W["v"]], xd)
+    o = rq.mul_mat(W["o"], q)
+    gate, up = rq.mul_mat_fused([W["gate"], W["up"]], o)
+    down = rq.mul_mat(W["down"], up)
+    torch.cuda.synchronize()
+    ref = lambda n, x: oracle.mul_mat(type_, blocks[n], x, 1.0, n_rot=shapes[n][0])
+    rq_, rk, rv = ref("q", x0), ref("k", x0), ref("v", x0)
+    ro = ref("o", rq_)
+    rg, ru = ref("gate", ro), ref("up", ro)
+    rd = ref("down", ru)
+    for name, got, want in [("q", q, rq_), ("k", k, rk), ("v", v, rv), ("o", o, ro), ("gate", gate, rg),
+                            ("up", up, ru), ("down", down, rd)]:
+        g = got.cpu().numpy()
+        assert bits_equal(g, want), name + ": " + first_mismatch(g, want)
+
+
+# ---------------------------------------------------------------- properties that hold at any size
+
+def test_rows_are_independent_and_calls_repeatable(oracle):
+    """A token's output must not depend on its neighbours or on the path taken (GEMV at M=1 vs GEMM inside M=300);
+    a second call with the same workspace must reproduce the first (split-K scratch left clean)."""
+    K, N, type_ = 5120, 1088, rq.TYPE_W4A4H
+    blocks = synth.random_weight_blocks(N, K, 7, type_, clip=0.9)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    x = synth.activations("student_t4", 300, K, 8)
+    xd = torch.from_numpy(x).to(DEV)
+    ws = W.workspace(300)
+    big = rq.mul_mat(W, xd, workspace=ws).clone()
+    again = rq.mul_mat(W, xd, workspace=ws).clone()
+    assert torch.equal(big, again)
+    for t in [0, 7, 131, 299]:
+        one = rq.mul_mat(W, xd[t:t + 1], workspace=ws)
+        assert torch.equal(one[0], big[t]), t
+    five = rq.mul_mat(W, xd[10:15], workspace=ws)
+    assert torch.equal(five, big[10:15])
