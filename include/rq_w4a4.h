@@ -8,7 +8,7 @@
  * Life cycle of one weight tensor, mirroring the reference's first-use / steady-state split
  * (P:2027-2075, P:295-299):
  *   first use   (may synchronize, must not be captured in a graph):
- *       read block 0's header on the host -> rq_w4a4_resolve_clip / rq_w4a4_rot_check;
+ *       read block 0's header on the host -> rq_w4a4_resolve_clip / rq_w4a4_tensor_rot;
  *       rq_w4a4_prepare() rewrites the 144-byte blocks into the streaming layout, OUT OF PLACE
  *       (the reference repacks in place and leaves the tensor unreadable as blocks; this does not).
  *   steady state (no allocation, no synchronization, no host reads: safe inside HIP graph capture):
@@ -99,6 +99,16 @@ int rq_w4a4_mul_mat(int type, const void *prepared_dev, int64_t K, int64_t N,
                     float *y_dev, int64_t ldy,
                     float clip, int64_t n_rot,
                     void *workspace_dev, size_t workspace_bytes, rq_stream_t stream);
+
+/* Measurement aid with no counterpart in the reference: rq_w4a4_mul_mat split into its two stages so that the
+ * product kernel can be timed alone. stages = 1: activation transform only (Hadamard + quantizer, also clears the
+ * split-K scratch); 2: product + epilogue only, on the workspace a previous stages-1 call filled for the same
+ * problem; 3: both (identical to rq_w4a4_mul_mat). */
+int rq_w4a4_mul_mat_stages(int type, const void *prepared_dev, int64_t K, int64_t N,
+                           const float *x_dev, int64_t ldx, int64_t M,
+                           float *y_dev, int64_t ldy,
+                           float clip, int64_t n_rot,
+                           void *workspace_dev, size_t workspace_bytes, rq_stream_t stream, int stages);
 
 /* Replaces ggml_cuda_mul_mat_rq_w4a4_fused (P:2371-2380): n <= 3 weights of one type, K, clip and rotation
  * length against the same x (q/k/v, gate/up): one activation transform, then one product per weight.

@@ -82,7 +82,7 @@ bool use_gemm(int64_t M) { return M >= env().gemm_min; }
 
 int run_products(int type, int n, const void *const *prepared, int64_t K, const int64_t *N, const float *x,
                  int64_t ldx, int64_t M, float *const *y, const int64_t *ldy, float clip, int64_t n_rot, void *ws,
-                 size_t ws_bytes, hipStream_t stream) {
+                 size_t ws_bytes, hipStream_t stream, int stages = 3) {
     if (n < 1 || n > 3 || !prepared || !N || !y || !ldy || !x || !ws) return RQ_E_ARGUMENT;
     int64_t Nmax = 0;
     for (int i = 0; i < n; ++i) {
@@ -124,8 +124,12 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
         q.zero_ptr = reinterpret_cast<int32_t *>(wsb + W.off_tot);
         q.zero_ints = (int64_t) ((W.bytes - W.off_tot) / sizeof(int32_t));
     }
-    hipError_t e = launch_rotate_quant(q, stream);
-    if (e != hipSuccess) return (int) e;
+    hipError_t e = hipSuccess;
+    if (stages & 1) {
+        e = launch_rotate_quant(q, stream);
+        if (e != hipSuccess) return (int) e;
+    }
+    if (!(stages & 2)) return 0;
 
     for (int i = 0; i < n; ++i) {
         const PreparedLayout L = prepared_layout(K, N[i]);
@@ -154,7 +158,6 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
                 g.ldy = ldy[i];
                 g.T = (int) (M - (int64_t) c * kGemvTokens < kGemvTokens ? M - (int64_t) c * kGemvTokens : kGemvTokens);
                 g.tot = reinterpret_cast<int32_t *>(wsb + W.off_tot);
-                g.cnt = reinterpret_cast<int32_t *>(wsb + W.off_cnt);
                 e = launch_gemv(g, stream);
                 if (e != hipSuccess) return (int) e;
             }
@@ -236,6 +239,14 @@ int rq_w4a4_mul_mat(int type, const void *prepared_dev, int64_t K, int64_t N, co
                     size_t workspace_bytes, rq_stream_t stream) {
     return run_products(type, 1, &prepared_dev, K, &N, x_dev, ldx, M, &y_dev, &ldy, clip, n_rot, workspace_dev,
                         workspace_bytes, (hipStream_t) stream);
+}
+
+int rq_w4a4_mul_mat_stages(int type, const void *prepared_dev, int64_t K, int64_t N, const float *x_dev, int64_t ldx,
+                           int64_t M, float *y_dev, int64_t ldy, float clip, int64_t n_rot, void *workspace_dev,
+                           size_t workspace_bytes, rq_stream_t stream, int stages) {
+    if (stages < 1 || stages > 3) return RQ_E_ARGUMENT;
+    return run_products(type, 1, &prepared_dev, K, &N, x_dev, ldx, M, &y_dev, &ldy, clip, n_rot, workspace_dev,
+                        workspace_bytes, (hipStream_t) stream, stages);
 }
 
 int rq_w4a4_mul_mat_fused(int type, int n, const void *const *prepared_dev, int64_t K, const int64_t *N,

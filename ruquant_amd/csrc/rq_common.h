@@ -63,7 +63,7 @@ inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
 //            tensor's nibble order) or the int8 form for the MFMA GEMM ([g][quarter][Mp][16 bytes], values q - z
 //            in the byte order the weight unpack produces).
 //   mz     : int4 form: [chunk][g][8] int32 = m | (8 - z) << 8 ... ; int8 form: [g][Mp] bytes = m.
-//   totals : split-K int32 sums [8 tokens][n_panels * 64] and one arrival counter per panel.
+//   totals : split-K cells [8 tokens][n_panels * 64], 64 bits each: arrival count above bit 48, exact sum below.
 // ---------------------------------------------------------------------------------------------------
 struct WorkspaceLayout {
     int64_t Mp;       // tokens padded to the GEMM tile
@@ -89,8 +89,8 @@ inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
     const size_t mz_i8 = (size_t) ng * W.Mp;
     W.off_mz = off;
     off = align_up(off + (mz_q4 > mz_i8 ? mz_q4 : mz_i8), 256);
-    W.tot_ints = (size_t) kGemvTokens * n_panels * kPanelRows;
-    W.cnt_ints = (size_t) n_panels;
+    W.tot_ints = (size_t) 2 * kGemvTokens * n_panels * kPanelRows;
+    W.cnt_ints = 0;
     W.off_tot = off;
     off = align_up(off + W.tot_ints * sizeof(int32_t), 256);
     W.off_cnt = off;
@@ -141,8 +141,7 @@ struct GemvArgs {
     float          *y;      // first token row of this chunk
     int64_t         ldy;
     int             T;      // 1..8 tokens
-    int32_t        *tot;    // split-K sums (zeroed)
-    int32_t        *cnt;    // arrival counters (zeroed)
+    int32_t        *tot;    // split-K cells (zero on entry, left zero)
 };
 hipError_t launch_gemv(const GemvArgs &a, hipStream_t stream);
 int gemv_ksplit(const PreparedLayout &L);

@@ -1,6 +1,6 @@
 // HBM-bound int4 x int4 GEMV for 1..8 tokens (decode and narrow verify widths) on gfx950.
 //
-// A workgroup of eight wavefronts owns one panel of 64 weight rows and one slice of K. Inside a wavefront
+// A workgroup of four wavefronts owns one panel of 64 weight rows and one slice of K. Inside a wavefront
 // lane = row: the prepared layout makes each group of 64 inputs two fully coalesced 1 KiB loads per
 // wavefront, the activation codes of that group are the same for all 64 lanes and arrive through scalar
 // loads, and v_dot8_i32_i4 consumes weight word x activation word directly. No lane ever exchanges data
@@ -18,67 +18,89 @@ namespace rq {
 
 namespace {
 
-constexpr int kWaves = 8;
-constexpr int kUnroll = 4;  // groups in flight per wavefront: 8 x 16-byte loads per lane
+constexpr int kGemvWaves = 4;
+constexpr int kUnroll = 5;  // groups in flight per wavefront: 10 x 16-byte loads per lane
 
 __device__ __forceinline__ int dot8(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot8((int) a, (int) b, c, false);
 }
 
-template <int T, bool HASK>
+// One batch = up to kUnroll groups of this wavefront. All weight loads of the batch are issued first; the
+// activation words of one token for the whole batch are fetched with scalar loads one token ahead of their use, so
+// their latency hides behind the weight loads (first token) or behind the previous token's arithmetic.
+template <int T, int kWaves>
 __device__ __forceinline__ void gemv_body(const uint4 *__restrict__ codes, const uint8_t *__restrict__ kmul,
                                           const uint32_t *__restrict__ act, const int32_t *__restrict__ mz,
-                                          int panel, int ng, int g_begin, int g_end, int wave, int lane,
-                                          int32_t (&tot)[T]) {
+                                          const int32_t *__restrict__ flags, int panel, int ng, int g_begin, int g_end,
+                                          int wave, int lane, int32_t (&tot)[T]) {
     const uint4 *wp = codes + (size_t) panel * ng * 128 + lane;
     const uint8_t *kp = kmul + (size_t) panel * ng * kPanelRows + lane;
     for (int g0 = g_begin + wave; g0 < g_end; g0 += kWaves * kUnroll) {
         uint4 q[kUnroll][2];
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const int g = min(g0 + k * kWaves, g_end - 1);  // past the end: reread the last group, contribute nothing
+            q[k][0] = wp[(size_t) g * 128];
+            q[k][1] = wp[(size_t) g * 128 + 64];
+        }
+        // (token, group) pairs in the order t * kUnroll + k; their activation words ride a ring of scalar
+        // registers kRing pairs deep
+        constexpr int kPairs = T * kUnroll;
+        constexpr int kRing = kPairs < 6 ? kPairs : 6;
+        uint32_t a[kRing][8];
+        int32_t mzv[kRing];
+        auto fetch_pair = [&](int j) {
+            const int t = j / kUnroll, k = j % kUnroll;
+            const int g = min(g0 + k * kWaves, g_end - 1);
+            const uint32_t *ap = act + ((size_t) g * kGemvTokens + t) * 8;  // wave-uniform address: scalar loads
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a[j % kRing][i] = ap[i];
+            mzv[j % kRing] = mz[(size_t) g * kGemvTokens + t];
+        };
+#pragma unroll
+        for (int j = 0; j < kRing - 1; ++j) fetch_pair(j);
+        // the multiplier flag is read here, after the weight loads are on their way (a volatile load cannot be
+        // hoisted in front of them)
+        const bool hask = *reinterpret_cast<const volatile int32_t *>(flags) & 1;
         int kw[kUnroll];
 #pragma unroll
         for (int k = 0; k < kUnroll; ++k) {
-            const int g = g0 + k * kWaves;
-            if (g < g_end) {
-                q[k][0] = wp[(size_t) g * 128];
-                q[k][1] = wp[(size_t) g * 128 + 64];
-                if (HASK) kw[k] = kp[(size_t) g * kPanelRows];
-            }
+            kw[k] = 1;
+            if (hask) kw[k] = kp[(size_t) min(g0 + k * kWaves, g_end - 1) * kPanelRows];
         }
+        int cs[kUnroll];
 #pragma unroll
         for (int k = 0; k < kUnroll; ++k) {
-            const int g = g0 + k * kWaves;
-            if (g < g_end) {
-                const uint32_t w[8] = { q[k][0].x, q[k][0].y, q[k][0].z, q[k][0].w,
-                                        q[k][1].x, q[k][1].y, q[k][1].z, q[k][1].w };
-                int cs = 0;
+            const uint32_t w[8] = { q[k][0].x, q[k][0].y, q[k][0].z, q[k][0].w, q[k][1].x, q[k][1].y, q[k][1].z, q[k][1].w };
+            int c = 0;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) cs = dot8(w[i], 0x11111111u, cs);
+            for (int i = 0; i < 8; ++i) c = dot8(w[i], 0x11111111u, c);
+            cs[k] = c;
+        }
 #pragma unroll
-                for (int t = 0; t < T; ++t) {
-                    const uint32_t *ap = act + ((size_t) g * kGemvTokens + t) * 8;  // wave-uniform: scalar loads
-                    int acc = 0;
+        for (int j = 0; j < kPairs; ++j) {
+            if (j + kRing - 1 < kPairs) fetch_pair(j + kRing - 1);
+            const int t = j / kUnroll, k = j % kUnroll, slot = j % kRing;
+            const uint32_t w[8] = { q[k][0].x, q[k][0].y, q[k][0].z, q[k][0].w, q[k][1].x, q[k][1].y, q[k][1].z, q[k][1].w };
+            int acc = 0;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) acc = dot8(w[i], ap[i], acc);
-                    const int32_t mzv = mz[(size_t) g * kGemvTokens + t];
-                    const int mult = mzv & 0xFF;
-                    const int zc = (int) (int8_t) ((mzv >> 8) & 0xFF);
-                    int term = mult * (acc + zc * cs);
-                    if (HASK) term *= kw[k];
-                    tot[t] += term >> kTermShift;
-                }
-            }
+            for (int i = 0; i < 8; ++i) acc = dot8(w[i], a[slot][i], acc);
+            const int mult = mzv[slot] & 0xFF;
+            const int zc = (int) (int8_t) ((mzv[slot] >> 8) & 0xFF);
+            int term = mult * (acc + zc * cs[k]);
+            if (hask) term *= kw[k];
+            if (g0 + k * kWaves < g_end) tot[t] += term >> kTermShift;
         }
     }
 }
 
-template <int T>
+template <int T, int kWaves>
 __global__ void __launch_bounds__(kWaves * 64)
 rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                const int32_t *__restrict__ flags, const uint32_t *__restrict__ act, const int32_t *__restrict__ mz,
                const float *__restrict__ u, float *__restrict__ y, int64_t ldy, int64_t N, int ng,
-               int32_t *__restrict__ tot_g, int32_t *__restrict__ cnt_g, int n_rows_pad) {
+               unsigned long long *__restrict__ cells, int n_rows_pad) {
     __shared__ int32_t red[kWaves][T][64];
-    __shared__ int s_last;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -91,73 +113,73 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
 #pragma unroll
     for (int t = 0; t < T; ++t) tot[t] = 0;
 
-    if (flags[0] & 1) {
-        gemv_body<T, true>(codes, kmul, act, mz, panel, ng, g_begin, g_end, wave, lane, tot);
-    } else {
-        gemv_body<T, false>(codes, kmul, act, mz, panel, ng, g_begin, g_end, wave, lane, tot);
-    }
+    gemv_body<T, kWaves>(codes, kmul, act, mz, flags, panel, ng, g_begin, g_end, wave, lane, tot);
 
 #pragma unroll
     for (int t = 0; t < T; ++t) red[wave][t][lane] = tot[t];
     __syncthreads();
 
-    const int64_t n = (int64_t) panel * kPanelRows + lane;
-    if (nks == 1) {
-        if (tid < T * 64) {
-            const int t = tid >> 6;
-            int32_t sum = 0;
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) sum += red[w][t][lane];
-            if (n < N) y[(int64_t) t * ldy + n] = (((float) sum * 16.0f) * u[t]) * s_w[n];
-        }
-        return;
-    }
-
-    // K is split over gridDim.y workgroups: exact int32 sums meet in global memory, the last arrival finishes
-    if (tid < T * 64) {
-        const int t = tid >> 6;
+    for (int item = tid; item < T * 64; item += kWaves * 64) {
+        const int t = item >> 6;
+        const int64_t n = (int64_t) panel * kPanelRows + lane;
         int32_t sum = 0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) sum += red[w][t][lane];
-        atomicAdd(&tot_g[(size_t) t * n_rows_pad + n], sum);
-    }
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) s_last = atomicAdd(&cnt_g[panel], 1) == nks - 1;
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    if (tid < T * 64) {
-        const int t = tid >> 6;
-        // read through the atomic unit (coherent across the chip) and leave the cell zero for the next pass
-        const int32_t sum = atomicExch(&tot_g[(size_t) t * n_rows_pad + n], 0);
+        if (nks > 1) {
+            // K is split over gridDim.y workgroups. Each output has one 64-bit cell: the low 48 bits collect the
+            // exact integer sum, the bits above count arrivals. One device-scope atomic add does both, and the
+            // value it returns tells the lane whether it was the last of the nks contributors; that lane alone
+            // finishes the output and clears the cell for the next call. No fences, no second round trip: the
+            // only cross-workgroup traffic is this one read-modify-write, performed in one place for the chip.
+            unsigned long long *cell = cells + (size_t) t * n_rows_pad + n;
+            const unsigned long long mine = (1ull << 48) + (unsigned long long) (long long) sum;
+            const unsigned long long now =
+                __hip_atomic_fetch_add(cell, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + mine;
+            if ((int) ((now + (1ull << 47)) >> 48) != nks) continue;
+            __hip_atomic_store(cell, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            sum = (int32_t) (uint32_t) now;  // the total fits int32 by construction of the format
+        }
         if (n < N) y[(int64_t) t * ldy + n] = (((float) sum * 16.0f) * u[t]) * s_w[n];
     }
-    if (tid == 0) atomicExch(&cnt_g[panel], 0);
+}
+
+template <int T, int kWaves>
+hipError_t launch_tw(const GemvArgs &a, int nks, hipStream_t stream) {
+    const uint8_t *p = a.prepared;
+    hipLaunchKernelGGL((rq_gemv_kernel<T, kWaves>), dim3(a.L.n_panels, nks), dim3(kWaves * 64), 0, stream,
+                       reinterpret_cast<const uint4 *>(p + a.L.off_codes),
+                       reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,
+                       reinterpret_cast<const int32_t *>(p + a.L.off_flags), a.act, a.mz, a.u, a.y, a.ldy, a.L.N,
+                       a.L.ng, reinterpret_cast<unsigned long long *>(a.tot), a.L.n_panels * kPanelRows);
+    return hipGetLastError();
 }
 
 template <int T>
 hipError_t launch_t(const GemvArgs &a, int nks, hipStream_t stream) {
-    const uint8_t *p = a.prepared;
-    hipLaunchKernelGGL((rq_gemv_kernel<T>), dim3(a.L.n_panels, nks), dim3(kWaves * 64), 0, stream,
-                       reinterpret_cast<const uint4 *>(p + a.L.off_codes),
-                       reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,
-                       reinterpret_cast<const int32_t *>(p + a.L.off_flags), a.act, a.mz, a.u, a.y, a.ldy, a.L.N,
-                       a.L.ng, a.tot, a.cnt, a.L.n_panels * kPanelRows);
-    return hipGetLastError();
+    static const int waves = getenv("RQ_GEMV_WAVES") ? atoi(getenv("RQ_GEMV_WAVES")) : kGemvWaves;
+    switch (waves) {
+        case 2:  return launch_tw<T, 2>(a, nks, stream);
+        case 8:  return launch_tw<T, 8>(a, nks, stream);
+        default: return launch_tw<T, 4>(a, nks, stream);
+    }
 }
 
 }  // namespace
 
-// How many workgroups share K for one panel: enough workgroups to cover the chip about twice, and at least
-// two groups per wavefront so the loads of a wavefront overlap.
+// How many workgroups share K for one panel. The kernel is a pure stream with a latency-bound start and end, so
+// it wants many small workgroups: their starts and tails overlap and the last wave of workgroups is short. Aim for
+// about a thousand workgroups, at least a batch (kGemvWaves x kUnroll groups) each when K allows, and never fewer
+// than four groups per workgroup.
 int gemv_ksplit(const PreparedLayout &L) {
     static const int forced = getenv("RQ_GEMV_KSPLIT") ? atoi(getenv("RQ_GEMV_KSPLIT")) : 0;
-    int nks = 1;
+    int nks;
     if (forced > 0) {
         nks = forced;
     } else {
-        while (L.n_panels * nks < 512 && L.ng / (nks * 2) >= kWaves * 2) nks *= 2;
+        const int by_batch = (L.ng + kGemvWaves * kUnroll - 1) / (kGemvWaves * kUnroll);
+        const int by_grid = (1024 + L.n_panels - 1) / L.n_panels;
+        nks = by_batch > by_grid ? by_batch : by_grid;
+        if (nks > L.ng / 4) nks = L.ng / 4;
     }
     if (nks > L.ng) nks = L.ng;
     return nks < 1 ? 1 : nks;

@@ -40,6 +40,10 @@ PROTOTYPES = {
                                        ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
                                        ctypes.c_int64, ctypes.c_float, ctypes.c_int64, ctypes.c_void_p,
                                        ctypes.c_size_t, ctypes.c_void_p]),
+    "rq_w4a4_mul_mat_stages": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                              ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
+                                              ctypes.c_int64, ctypes.c_float, ctypes.c_int64, ctypes.c_void_p,
+                                              ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int]),
     "rq_w4a4_mul_mat_fused": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_void_p),
                                              ctypes.c_int64, c_i64p, ctypes.c_void_p, ctypes.c_int64,
                                              ctypes.c_int64, ctypes.POINTER(ctypes.c_void_p), c_i64p,
