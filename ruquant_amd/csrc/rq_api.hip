@@ -138,7 +138,6 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
             g.L = L;
             g.act8 = wsb + W.off_act;
-            g.m8 = wsb + W.off_mz;
             g.u = q.u;
             g.y = y[i];
             g.ldy = ldy[i];

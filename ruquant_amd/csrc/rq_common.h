@@ -60,9 +60,9 @@ inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
 //
 //   u      : Mp floats, the token units.
 //   act    : either the int4 form for the GEMV  ([chunk][g][8 token slots][8 words], codes q - 8, the
-//            tensor's nibble order) or the int8 form for the MFMA GEMM ([g][quarter][Mp][16 bytes], values q - z
-//            in the byte order the weight unpack produces).
-//   mz     : int4 form: [chunk][g][8] int32 = m | (8 - z) << 8 ... ; int8 form: [g][Mp] bytes = m.
+//            tensor's nibble order) or the int8 form for the MFMA GEMM ([g][digit][quarter][Mp][16 bytes]: the two
+//            balanced digits of m (q - z), in the byte order the weight unpack produces).
+//   mz     : int4 form only: [chunk][g][8] int32 = m | (8 - z) << 8.
 //   totals : split-K cells [8 tokens][n_panels * 64], 64 bits each: arrival count above bit 48, exact sum below.
 // ---------------------------------------------------------------------------------------------------
 struct WorkspaceLayout {
@@ -82,11 +82,11 @@ inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
     W.off_u = off;
     off = align_up(off + (size_t) (W.Mp > (int64_t) W.chunks * 8 ? W.Mp : (int64_t) W.chunks * 8) * sizeof(float), 256);
     const size_t act_q4 = (size_t) W.chunks * ng * kGemvTokens * 32;
-    const size_t act_i8 = (size_t) ng * W.Mp * 64;
+    const size_t act_i8 = (size_t) ng * W.Mp * 128;
     W.off_act = off;
     off = align_up(off + (act_q4 > act_i8 ? act_q4 : act_i8), 256);
     const size_t mz_q4 = (size_t) W.chunks * ng * kGemvTokens * sizeof(int32_t);
-    const size_t mz_i8 = (size_t) ng * W.Mp;
+    const size_t mz_i8 = 0;
     W.off_mz = off;
     off = align_up(off + (mz_q4 > mz_i8 ? mz_q4 : mz_i8), 256);
     W.tot_ints = (size_t) 2 * kGemvTokens * n_panels * kPanelRows;
@@ -104,7 +104,7 @@ enum ActMode : int {
     kActRotateOnly = 0,  // fp32 rotated rows (rq_w4a4_hadamard)
     kActBlocks     = 1,  // the reference's A4 / A4H block rows (rq_w4a4_quantize_act)
     kActQ4         = 2,  // int4 codes + (m, 8 - z) words for the GEMV
-    kActI8         = 3,  // int8 (q - z) + m bytes for the MFMA GEMM
+    kActI8         = 3,  // two int8 digits of m (q - z) for the MFMA GEMM
 };
 
 struct RotQuantArgs {
@@ -149,8 +149,7 @@ int gemv_ksplit(const PreparedLayout &L);
 struct GemmArgs {
     const uint8_t  *prepared;
     PreparedLayout  L;
-    const uint8_t  *act8;   // [g][quarter][Mp][16]
-    const uint8_t  *m8;     // [g][Mp]
+    const uint8_t  *act8;   // [g][digit][quarter][Mp][16]
     const float    *u;      // [Mp]
     float          *y;
     int64_t         ldy;

@@ -237,18 +237,29 @@ __global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs
         for (int j = 0; j < 8; ++j) q[j] = (int) fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
 
         if (a.mode == kActI8) {
-            // bytes q - z in the order the weight unpack yields: even codes of the word, then odd codes
-            uint32_t lo4 = 0, hi4 = 0;
+            // p = m (q - z), |p| <= 3825, as two balanced int8 digits p = 64 hi + lo, lo in [-32, 31]; bytes in the
+            // order the weight unpack yields: the even codes of the word, then the odd codes
+            uint32_t lo_e = 0, lo_o = 0, hi_e = 0, hi_o = 0;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                lo4 |= (uint32_t) ((q[2 * j] - z) & 0xFF) << (8 * j);
-                hi4 |= (uint32_t) ((q[2 * j + 1] - z) & 0xFF) << (8 * j);
+            for (int j = 0; j < 8; ++j) {
+                const int p = mg * (q[j] - z);
+                const int lo = ((p + 32) & 63) - 32;
+                const int hi = (p - lo) >> 6;
+                const int sh = 8 * (j >> 1);
+                if (j & 1) {
+                    lo_o |= (uint32_t) (lo & 0xFF) << sh;
+                    hi_o |= (uint32_t) (hi & 0xFF) << sh;
+                } else {
+                    lo_e |= (uint32_t) (lo & 0xFF) << sh;
+                    hi_e |= (uint32_t) (hi & 0xFF) << sh;
+                }
             }
             if (on) {
-                // [group][quarter of the group][token][16 bytes]: a token tile of one quarter is contiguous
-                uint32_t *dst = a.act + (((size_t) g * 4 + ((w & 7) >> 1)) * a.Mp + t) * 4 + (w & 1) * 2;
-                *reinterpret_cast<uint2 *>(dst) = make_uint2(lo4, hi4);
-                if ((tid & 7) == 0) reinterpret_cast<uint8_t *>(a.mz)[(size_t) g * a.Mp + t] = (uint8_t) mg;
+                // [group][digit][quarter of the group][token][16 bytes]: a token tile of one quarter is contiguous
+                const size_t cell = (((size_t) g * 2 + 0) * 4 + ((w & 7) >> 1)) * a.Mp + t;
+                uint32_t *dst = a.act + cell * 4 + (w & 1) * 2;
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(lo_e, lo_o);
+                *reinterpret_cast<uint2 *>(dst + (size_t) 16 * a.Mp) = make_uint2(hi_e, hi_o);
             }
             continue;
         }
