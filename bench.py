@@ -152,6 +152,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy 10 times (scale for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--shapes", default="", help="comma-separated names of the extra shapes to run (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -165,6 +167,14 @@ def main():
         sys.exit(1)
     import ruquant_amd as rq
     rq.load_library()   # fails loudly when the HIP library has not been built
+
+    if args.copy_calibration:
+        src = torch.ones(64 << 20, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            torch.mul(src, 1.0, out=dst)     # a plain elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     K, N, M = 5120, 17408, 1
     head = Problem(K, N, M, "outlier_channels", 0.9, seed=2)

@@ -108,18 +108,44 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint
             for (int i = 0; i < 4; ++i) kk[rt][i] = (k4 >> (8 * i)) & 0xFF;
         }
     }
+    if (!HASK) {
+        // Software pipeline over the four token tiles: the eight MFMAs of tile ct are issued back to back while the
+        // vector ALU folds the four results of tile ct - 1, so neither unit waits for the other.
+        v4i S[2][4];
 #pragma unroll
-    for (int ct = 0; ct < 4; ++ct) {
-        const v4i Blo = as_v4i(s.b[0][c.quad][64 * c.wc + 16 * ct + c.l16]);
-        const v4i Bhi = as_v4i(s.b[1][c.quad][64 * c.wc + 16 * ct + c.l16]);
+        for (int ct = 0; ct < 5; ++ct) {
+            if (ct < 4) {
+                const v4i Blo = as_v4i(s.b[0][c.quad][64 * c.wc + 16 * ct + c.l16]);
+                const v4i Bhi = as_v4i(s.b[1][c.quad][64 * c.wc + 16 * ct + c.l16]);
 #pragma unroll
-        for (int rt = 0; rt < 4; ++rt) {
-            if (!HASK) {
-                hi[rt][ct] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Bhi, hi[rt][ct], 0, 0, 0);
-                const v4i S = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Blo, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+                for (int rt = 0; rt < 4; ++rt) {
+                    S[ct & 1][rt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Blo, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+                    hi[rt][ct] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Bhi, hi[rt][ct], 0, 0, 0);
+                }
+            }
+            if (ct > 0) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) lo[rt][ct][i] += S[i] >> 8;
-            } else {
+                for (int rt = 0; rt < 4; ++rt) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) lo[rt][ct - 1][i] += S[(ct - 1) & 1][rt][i] >> 8;
+                }
+            }
+            if (ct > 0 && ct < 4) {
+                // 8 MFMAs interleaved with the 32 vector ops of the previous tile's fold: 1 MFMA, 4 VALU, ...
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // VALU
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+            const v4i Blo = as_v4i(s.b[0][c.quad][64 * c.wc + 16 * ct + c.l16]);
+            const v4i Bhi = as_v4i(s.b[1][c.quad][64 * c.wc + 16 * ct + c.l16]);
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
                 const v4i H = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Bhi, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
                 const v4i S = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Blo, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
 #pragma unroll
