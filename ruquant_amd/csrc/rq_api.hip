@@ -122,7 +122,9 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     q.Mp = (int) W.Mp;
     if (!gemm) {
         q.zero_ptr = reinterpret_cast<int32_t *>(wsb + W.off_tot);
-        q.zero_ints = (int64_t) ((W.bytes - W.off_tot) / sizeof(int32_t));
+        // only the token slots this call can touch: [min(M, 8)][padded rows] cells of two ints
+        const int64_t slots = M < kGemvTokens ? M : kGemvTokens;
+        q.zero_ints = 2 * slots * (int64_t) ((Nmax + kPanelRows - 1) / kPanelRows * kPanelRows);
     }
     hipError_t e = hipSuccess;
     if (stages & 1) {

@@ -1,0 +1,133 @@
+#include "rq_ggml_adapter.h"
+
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+namespace {
+
+// what the reference keeps per weight after its first use (rq_tensor_info, P:1820-1826)
+struct rq_first_use {
+    float   clip;
+    int64_t n_rot;
+    void   *prepared;
+    size_t  prepared_bytes;
+};
+
+[[noreturn]] void rq_abort(const char *what, long long a = 0, long long b = 0) {
+    fprintf(stderr, "ruquant W4A4: %s (%lld, %lld)\n", what, a, b);
+    abort();
+}
+
+void hip_check(hipError_t e, const char *what) {
+    if (e != hipSuccess) {
+        fprintf(stderr, "ruquant W4A4: %s: %s\n", what, hipGetErrorString(e));
+        abort();
+    }
+}
+
+bool is_rq_type(int t) { return t == RQ_GGML_TYPE_W4A4 || t == RQ_GGML_TYPE_W4A4H; }
+
+bool contiguous_blocks(const rq_tensor *t) {
+    const size_t row = (size_t) (t->ne[0] / RQ_BLOCK_CODES) * RQ_BLOCK_BYTES;
+    return t->nb[0] == RQ_BLOCK_BYTES && t->nb[1] == row;
+}
+
+// first use, never inside a graph capture: read block 0's header, resolve clip and rotation length, prepare
+rq_first_use *first_use(rq_backend_context &ctx, const rq_tensor *src0) {
+    if (src0->extra) return (rq_first_use *) src0->extra;
+    rq_block_w4a4 hdr;
+    hipStream_t stream = (hipStream_t) ctx.stream;
+    hip_check(hipMemcpyAsync(&hdr, src0->data, 16, hipMemcpyDeviceToHost, stream), "header read");
+    hip_check(hipStreamSynchronize(stream), "header read");
+    rq_first_use *fu = new rq_first_use;
+    fu->clip = rq_w4a4_resolve_clip(&hdr, src0->type);
+    fu->n_rot = rq_w4a4_tensor_rot(&hdr, src0->type, src0->ne[0]);
+    if (fu->n_rot < 0) {
+        rq_abort("W4A4H: Hadamard length does not divide this row slice (ruquant convert --rot-blocks)", hdr.pad[0],
+                 src0->ne[0]);
+    }
+    fu->prepared_bytes = rq_w4a4_prepared_bytes(src0->ne[0], src0->ne[1]);
+    hip_check(hipMalloc(&fu->prepared, fu->prepared_bytes), "prepared weight");
+    const int rc = rq_w4a4_prepare(src0->data, src0->ne[0], src0->ne[1], fu->prepared, fu->prepared_bytes, ctx.stream);
+    if (rc != 0) rq_abort("rq_w4a4_prepare failed", rc);
+    const_cast<rq_tensor *>(src0)->extra = fu;
+    return fu;
+}
+
+void *scratch(rq_backend_context &ctx, size_t bytes) {
+    if (ctx.scratch_bytes < bytes) {
+        // growing is a first-use event too: let the stream drain before the old buffer goes away
+        hip_check(hipStreamSynchronize((hipStream_t) ctx.stream), "scratch");
+        if (ctx.scratch) hip_check(hipFree(ctx.scratch), "scratch");
+        hip_check(hipMalloc(&ctx.scratch, bytes), "scratch");
+        ctx.scratch_bytes = bytes;
+    }
+    return ctx.scratch;
+}
+
+}  // namespace
+
+rq_backend_context::~rq_backend_context() {
+    if (scratch) (void) hipFree(scratch);
+}
+
+bool ggml_cuda_rq_w4a4_supported(int cc, const rq_tensor *src0, const rq_tensor *src1, const rq_tensor *dst) {
+    (void) cc;
+    return is_rq_type(src0->type) && src1->type == RQ_GGML_TYPE_F32 && dst->type == RQ_GGML_TYPE_F32 &&
+           src0->ne[2] == 1 && src0->ne[3] == 1 && src1->ne[2] == 1 && src1->ne[3] == 1 && contiguous_blocks(src0) &&
+           src1->nb[0] == sizeof(float) && dst->nb[0] == sizeof(float) && src1->ne[0] == src0->ne[0] &&
+           rq_w4a4_supported(src0->type, src0->ne[0], src0->ne[1], src1->ne[1], (int64_t) src1->nb[1],
+                             (int64_t) dst->nb[1]) != 0;
+}
+
+bool ggml_cuda_rq_w4a4_ready(const rq_tensor *src0) { return src0->extra != nullptr; }
+
+void ggml_cuda_mul_mat_rq_w4a4_fused(rq_backend_context &ctx, const rq_tensor *const *src0s, rq_tensor *const *dsts, int n,
+                                     const rq_tensor *src1) {
+    if (n < 1 || n > 3) rq_abort("fused call takes 1..3 weights", n);
+    const void *prepared[3];
+    float *ys[3];
+    int64_t Ns[3], ldys[3];
+    const rq_first_use *fu0 = nullptr;
+    int64_t Nmax = 0;
+    for (int i = 0; i < n; ++i) {
+        const rq_first_use *fu = first_use(ctx, src0s[i]);
+        if (i == 0) fu0 = fu;
+        if (src0s[i]->type != src0s[0]->type || src0s[i]->ne[0] != src0s[0]->ne[0] || fu->clip != fu0->clip ||
+            fu->n_rot != fu0->n_rot) {
+            rq_abort("fused weights must share type, K, clip and rotation length");
+        }
+        prepared[i] = fu->prepared;
+        ys[i] = (float *) dsts[i]->data;
+        Ns[i] = src0s[i]->ne[1];
+        ldys[i] = (int64_t) (dsts[i]->nb[1] / sizeof(float));
+        if (Ns[i] > Nmax) Nmax = Ns[i];
+    }
+    const int64_t K = src0s[0]->ne[0], M = src1->ne[1];
+    const size_t ws_bytes = rq_w4a4_workspace_bytes(src0s[0]->type, K, Nmax, M);
+    void *ws = scratch(ctx, ws_bytes);
+    const int rc = rq_w4a4_mul_mat_fused(src0s[0]->type, n, prepared, K, Ns, (const float *) src1->data,
+                                         (int64_t) (src1->nb[1] / sizeof(float)), M, ys, ldys, fu0->clip, fu0->n_rot, ws,
+                                         ws_bytes, ctx.stream);
+    if (rc != 0) rq_abort("no path for this shape", rc);   // the reference: GGML_ABORT (P:2337)
+}
+
+void ggml_cuda_mul_mat_rq_w4a4(rq_backend_context &ctx, const rq_tensor *src0, const rq_tensor *src1, rq_tensor *dst) {
+    ggml_cuda_mul_mat_rq_w4a4_fused(ctx, &src0, &dst, 1, src1);
+}
+
+bool ggml_cuda_rq_w4a4_can_fuse(const rq_tensor *a, const rq_tensor *b) {
+    if (a->op != RQ_GGML_OP_MUL_MAT || b->op != RQ_GGML_OP_MUL_MAT) return false;
+    const rq_tensor *wa = a->src[0], *wb = b->src[0], *x = a->src[1];
+    if (b->src[1] != x || !is_rq_type(wa->type) || wb->type != wa->type || wb->ne[0] != wa->ne[0] ||
+        x->type != RQ_GGML_TYPE_F32 || x->ne[2] != 1 || x->ne[3] != 1 || x->ne[1] > 16 ||
+        a->type != RQ_GGML_TYPE_F32 || b->type != RQ_GGML_TYPE_F32) {
+        return false;
+    }
+    // both weights seen before: a first use synchronizes, so it stays unfused
+    const rq_first_use *ia = (const rq_first_use *) wa->extra, *ib = (const rq_first_use *) wb->extra;
+    return ia != nullptr && ib != nullptr && ia->clip == ib->clip && ia->n_rot == ib->n_rot;
+}
+
+void ggml_cuda_rq_graph_begin(rq_backend_context &ctx) { (void) ctx; }
