@@ -51,6 +51,7 @@ struct Env {
         const char *gm = getenv("RQ_GEMM_MIN");
         gemm_min = gm ? atoi(gm) : 33;
         if (gemm_min < 1) gemm_min = 1;
+        if (gemm_min > kGemvMaxTokens + 1) gemm_min = kGemvMaxTokens + 1;
     }
 };
 
@@ -115,12 +116,21 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     q.m = m;
     q.scale = 1.0f / sqrtf((float) q.n_rot);
     q.clip = clip;
-    q.mode = gemm ? kActI8 : kActQ4;
+    q.mode = gemm ? kActI8 : kActStats;
     q.u = reinterpret_cast<float *>(wsb + W.off_u);
     q.act = reinterpret_cast<uint32_t *>(wsb + W.off_act);
-    q.mz = wsb + W.off_mz;
     q.Mp = (int) W.Mp;
+    const float *gemv_x = x;      // what the GEMV quantizes from: the rotated rows, or x itself for W4A4
+    int64_t gemv_ldx = ldx;
     if (!gemm) {
+        q.lohi = reinterpret_cast<float *>(wsb + W.off_lohi);
+        q.rpart = reinterpret_cast<float *>(wsb + W.off_rpart);
+        if (q.rotate) {
+            q.out_f32 = reinterpret_cast<float *>(wsb + W.off_act);
+            q.ldo = K;
+            gemv_x = q.out_f32;
+            gemv_ldx = K;
+        }
         q.zero_ptr = reinterpret_cast<int32_t *>(wsb + W.off_tot);
         // only the token slots this call can touch: [min(M, 8)][padded rows] cells of two ints
         const int64_t slots = M < kGemvTokens ? M : kGemvTokens;
@@ -128,7 +138,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     }
     hipError_t e = hipSuccess;
     if (stages & 1) {
-        e = launch_rotate_quant(q, stream);
+        e = gemm ? launch_rotate_quant(q, stream) : launch_rotate_stats(q, stream);
         if (e != hipSuccess) return (int) e;
     }
     if (!(stages & 2)) return 0;
@@ -152,9 +162,10 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
                 GemvArgs g;
                 g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
                 g.L = L;
-                g.act = q.act + (size_t) c * L.ng * kGemvTokens * 8;
-                g.mz = reinterpret_cast<const int32_t *>(wsb + W.off_mz) + (size_t) c * L.ng * kGemvTokens;
-                g.u = q.u + c * kGemvTokens;
+                g.x = gemv_x + (int64_t) c * kGemvTokens * gemv_ldx;
+                g.ldx = gemv_ldx;
+                g.lohi = q.lohi + (size_t) c * kGemvTokens * L.ng * 2;
+                g.rpart = q.rpart + (size_t) c * kGemvTokens * kRangeParts;
                 g.y = y[i] + (int64_t) c * kGemvTokens * ldy[i];
                 g.ldy = ldy[i];
                 g.T = (int) (M - (int64_t) c * kGemvTokens < kGemvTokens ? M - (int64_t) c * kGemvTokens : kGemvTokens);

@@ -14,6 +14,8 @@ constexpr int kPanelRows  = 64;   // weight rows per panel: one wavefront lane p
 constexpr int kTermShift  = 4;    // RQ_TERM_SHIFT (reference patch line 39)
 constexpr int kGemvTokens = 8;    // tokens per GEMV pass; the activation slot stride of the int4 layout
 constexpr int kGemmTokens = 128;  // token tile of the MFMA GEMM; int8 activations are padded to it
+constexpr int kRangeParts = 32;    // partial maxima of a token's group ranges handed from the activation kernel to the GEMV
+constexpr int kGemvMaxTokens = 64;  // the dispatcher never sends more tokens than this down the GEMV path
 
 // ---------------------------------------------------------------------------------------------------
 // Prepared weight (written once by rq_w4a4_prepare, read by every product kernel).
@@ -58,18 +60,19 @@ inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
 // ---------------------------------------------------------------------------------------------------
 // Workspace of one rq_w4a4_mul_mat call.
 //
-//   u      : Mp floats, the token units.
-//   act    : either the int4 form for the GEMV  ([chunk][g][8 token slots][8 words], codes q - 8, the
-//            tensor's nibble order) or the int8 form for the MFMA GEMM ([g][digit][quarter][Mp][16 bytes]: the two
-//            balanced digits of m (q - z), in the byte order the weight unpack produces).
-//   mz     : int4 form only: [chunk][g][8] int32 = m | (8 - z) << 8.
-//   totals : split-K cells [8 tokens][n_panels * 64], 64 bits each: arrival count above bit 48, exact sum below.
+//   u      : Mp floats, the token units (GEMM path; the GEMV derives them itself).
+//   act    : GEMV path (M <= 32): the rotated activations as fp32 rows [M][K] followed by the clipped group
+//            ranges [M][ng][2] (lo, hi) and [M][32] partial maxima of hi - lo; every GEMV workgroup quantizes
+//            the K slice it consumes itself.
+//            GEMM path: two int8 digit planes of m (q - z), [g][digit][quarter][Mp][16 bytes], in the byte order
+//            the weight unpack produces.
+//   cells  : split-K cells [8 tokens][n_panels * 64], 64 bits each: arrival count above bit 48, exact sum below.
 // ---------------------------------------------------------------------------------------------------
 struct WorkspaceLayout {
     int64_t Mp;       // tokens padded to the GEMM tile
     int     chunks;   // ceil(M / 8)
-    size_t  off_u, off_act, off_mz, off_tot, off_cnt, bytes;
-    size_t  tot_ints, cnt_ints;
+    size_t  off_u, off_act, off_lohi, off_rpart, off_tot, bytes;
+    size_t  tot_ints;
 };
 
 inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
@@ -80,21 +83,20 @@ inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
     W.chunks = (int) ((M + kGemvTokens - 1) / kGemvTokens);
     size_t off = 0;
     W.off_u = off;
-    off = align_up(off + (size_t) (W.Mp > (int64_t) W.chunks * 8 ? W.Mp : (int64_t) W.chunks * 8) * sizeof(float), 256);
-    const size_t act_q4 = (size_t) W.chunks * ng * kGemvTokens * 32;
-    const size_t act_i8 = (size_t) ng * W.Mp * 128;
+    off = align_up(off + (size_t) W.Mp * sizeof(float), 256);
+    const size_t rows = (size_t) M * K * sizeof(float);          // GEMV form (only taken for small M)
+    const size_t lohi = (size_t) M * ng * 2 * sizeof(float);
+    const size_t act_i8 = (size_t) ng * W.Mp * 128;              // GEMM form
+    const bool small = M <= kGemvMaxTokens;
     W.off_act = off;
-    off = align_up(off + (act_q4 > act_i8 ? act_q4 : act_i8), 256);
-    const size_t mz_q4 = (size_t) W.chunks * ng * kGemvTokens * sizeof(int32_t);
-    const size_t mz_i8 = 0;
-    W.off_mz = off;
-    off = align_up(off + (mz_q4 > mz_i8 ? mz_q4 : mz_i8), 256);
+    W.off_lohi = off + align_up(rows, 256);
+    const size_t rpart = (size_t) M * kRangeParts * sizeof(float);
+    W.off_rpart = W.off_lohi + align_up(lohi, 256);
+    const size_t gemv_form = align_up(rows, 256) + align_up(lohi, 256) + align_up(rpart, 256);
+    off = align_up(off + (small && gemv_form > act_i8 ? gemv_form : act_i8), 256);
     W.tot_ints = (size_t) 2 * kGemvTokens * n_panels * kPanelRows;
-    W.cnt_ints = 0;
     W.off_tot = off;
     off = align_up(off + W.tot_ints * sizeof(int32_t), 256);
-    W.off_cnt = off;
-    off = align_up(off + W.cnt_ints * sizeof(int32_t), 256);
     W.bytes = off;
     return W;
 }
@@ -103,7 +105,7 @@ inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
 enum ActMode : int {
     kActRotateOnly = 0,  // fp32 rotated rows (rq_w4a4_hadamard)
     kActBlocks     = 1,  // the reference's A4 / A4H block rows (rq_w4a4_quantize_act)
-    kActQ4         = 2,  // int4 codes + (m, 8 - z) words for the GEMV
+    kActStats      = 2,  // fp32 (rotated) rows + clipped group ranges for the GEMV, which quantizes its own slice
     kActI8         = 3,  // two int8 digits of m (q - z) for the MFMA GEMM
 };
 
@@ -117,12 +119,13 @@ struct RotQuantArgs {
     float        clip;
     int          mode;
     // outputs
-    float       *out_f32;  int64_t ldo;   // kActRotateOnly
+    float       *out_f32;  int64_t ldo;   // kActRotateOnly, kActStats (may be null when rotate == 0)
+    float       *lohi;                    // kActStats: [M][K / 64][2]
+    float       *rpart;                   // kActStats: [M][kRangeParts] partial maxima of hi - lo (max of them = R)
     void        *blocks;                  // kActBlocks
     int32_t      len_field;               // kActBlocks: pad[1] of the activation blocks (K or n_rot)
     float       *u;
-    uint32_t    *act;                     // kActQ4 / kActI8
-    void        *mz;
+    uint32_t    *act;                     // kActI8
     int          Mp;                      // kActI8: padded token count (rows M..Mp-1 are zero filled)
     // split-K scratch to clear (blocks past the token blocks do it)
     int32_t     *zero_ptr;
@@ -132,12 +135,17 @@ struct RotQuantArgs {
 
 hipError_t launch_rotate_quant(const RotQuantArgs &a, hipStream_t stream);
 
+// Activation side of the GEMV path: like launch_rotate_quant with mode kActStats, but spreads one token over
+// several workgroups when the rotation allows it (decode latency).
+hipError_t launch_rotate_stats(const RotQuantArgs &a, hipStream_t stream);
+
 struct GemvArgs {
     const uint8_t  *prepared;
     PreparedLayout  L;
-    const uint32_t *act;    // int4 activation form of this chunk
-    const int32_t  *mz;
-    const float    *u;      // units of this chunk's tokens
+    const float    *x;      // (rotated) activations of this chunk's first token
+    int64_t         ldx;    // row stride in floats
+    const float    *lohi;   // clipped group ranges of this chunk's first token, [T][ng][2]
+    const float    *rpart;  // partial range maxima of this chunk's first token, [T][kRangeParts]
     float          *y;      // first token row of this chunk
     int64_t         ldy;
     int             T;      // 1..8 tokens

@@ -2,10 +2,17 @@
 //
 // A workgroup of four wavefronts owns one panel of 64 weight rows and one slice of K. Inside a wavefront
 // lane = row: the prepared layout makes each group of 64 inputs two fully coalesced 1 KiB loads per
-// wavefront, the activation codes of that group are the same for all 64 lanes and arrive through scalar
-// loads, and v_dot8_i32_i4 consumes weight word x activation word directly. No lane ever exchanges data
-// with another lane until the per-wave totals meet in LDS. The per-group fold, the exact int32 total and
-// the fp32 epilogue are those of ggml_vec_dot_w4a4_a4 (reference patch lines 148-177):
+// wavefront, and v_dot8_i32_i4 consumes weight word x activation word directly. No lane exchanges data with another
+// lane until the per-wave totals meet in LDS.
+//
+// The activation quantizer is part of this kernel. Its inputs are the (rotated) fp32 rows and the clipped range of
+// every 64-wide group; a workgroup first puts the weight loads of its first batch in flight, then derives the
+// token units from all ranges (reference patch lines 2646-2655: R = widest range, u = R / 3825), quantizes just the
+// groups of its own K slice into LDS (lines 2662-2677: m, 1 / (m u), z, q, op for op) and meets its weights. So
+// the quantizer costs no launch, no trip through memory for the codes, and its latency hides behind the first
+// weight loads.
+//
+// The per-group fold, the exact int32 total and the fp32 epilogue are those of ggml_vec_dot_w4a4_a4 (lines 148-177):
 //     total += (k * m_g * (acc_g + (8 - z_g) * colsum_g)) >> 4;   y = ((float(total) * 16) * u) * s_w.
 // colsum_g is recomputed from the codes (dot8 against 0x11111111) instead of being stored.
 #include "rq_common.h"
@@ -19,77 +26,68 @@ namespace rq {
 namespace {
 
 constexpr int kGemvWaves = 4;
-constexpr int kUnroll = 5;  // groups in flight per wavefront: 10 x 16-byte loads per lane
+constexpr int kUnroll = 5;        // groups in flight per wavefront: 10 x 16-byte loads per lane
+constexpr int kMaxSlice = 48;     // most groups one workgroup may own (bounds its LDS)
 
 __device__ __forceinline__ int dot8(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot8((int) a, (int) b, c, false);
 }
 
-// One batch = up to kUnroll groups of this wavefront. All weight loads of the batch are issued first; the
-// activation words of one token for the whole batch are fetched with scalar loads one token ahead of their use, so
-// their latency hides behind the weight loads (first token) or behind the previous token's arithmetic.
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+struct Batch {
+    uint4 q[kUnroll][2];
+};
+
+template <int kWaves>
+__device__ __forceinline__ void load_batch(Batch &b, const uint4 *wp, int g0, int g_end) {
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+        const int g = min(g0 + k * kWaves, g_end - 1);  // past the end: reread the last group, contribute nothing
+        b.q[k][0] = wp[(size_t) g * 128];
+        b.q[k][1] = wp[(size_t) g * 128 + 64];
+    }
+}
+
+// act: [group of the slice][token][8 words] codes q - 8 in the tensor's nibble order; mz: m | (8 - z) << 8
 template <int T, int kWaves>
-__device__ __forceinline__ void gemv_body(const uint4 *__restrict__ codes, const uint8_t *__restrict__ kmul,
-                                          const uint32_t *__restrict__ act, const int32_t *__restrict__ mz,
-                                          const int32_t *__restrict__ flags, int panel, int ng, int g_begin, int g_end,
-                                          int wave, int lane, int32_t (&tot)[T]) {
-    const uint4 *wp = codes + (size_t) panel * ng * 128 + lane;
-    const uint8_t *kp = kmul + (size_t) panel * ng * kPanelRows + lane;
-    for (int g0 = g_begin + wave; g0 < g_end; g0 += kWaves * kUnroll) {
-        uint4 q[kUnroll][2];
+__device__ __forceinline__ void compute_batch(const Batch &b, const uint8_t *kp, bool hask, const uint32_t *act,
+                                              const int32_t *mz, int g0, int g_begin, int g_end, int32_t (&tot)[T]) {
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
-            const int g = min(g0 + k * kWaves, g_end - 1);  // past the end: reread the last group, contribute nothing
-            q[k][0] = wp[(size_t) g * 128];
-            q[k][1] = wp[(size_t) g * 128 + 64];
-        }
-        // (token, group) pairs in the order t * kUnroll + k; their activation words ride a ring of scalar
-        // registers kRing pairs deep
-        constexpr int kPairs = T * kUnroll;
-        constexpr int kRing = kPairs < 6 ? kPairs : 6;
-        uint32_t a[kRing][8];
-        int32_t mzv[kRing];
-        auto fetch_pair = [&](int j) {
-            const int t = j / kUnroll, k = j % kUnroll;
-            const int g = min(g0 + k * kWaves, g_end - 1);
-            const uint32_t *ap = act + ((size_t) g * kGemvTokens + t) * 8;  // wave-uniform address: scalar loads
+    for (int k = 0; k < kUnroll; ++k) {
+        const int g = g0 + k * kWaves;
+        if (g >= g_end) break;   // wave-uniform
+        const uint32_t w[8] = { b.q[k][0].x, b.q[k][0].y, b.q[k][0].z, b.q[k][0].w,
+                                b.q[k][1].x, b.q[k][1].y, b.q[k][1].z, b.q[k][1].w };
+        int cs = 0;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) a[j % kRing][i] = ap[i];
-            mzv[j % kRing] = mz[(size_t) g * kGemvTokens + t];
-        };
+        for (int i = 0; i < 8; ++i) cs = dot8(w[i], 0x11111111u, cs);
+        int kw = 1;
+        if (hask) kw = kp[(size_t) g * kPanelRows];
+        const int gl = g - g_begin;
 #pragma unroll
-        for (int j = 0; j < kRing - 1; ++j) fetch_pair(j);
-        // the multiplier flag is read here, after the weight loads are on their way (a volatile load cannot be
-        // hoisted in front of them)
-        const bool hask = *reinterpret_cast<const volatile int32_t *>(flags) & 1;
-        int kw[kUnroll];
-#pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
-            kw[k] = 1;
-            if (hask) kw[k] = kp[(size_t) min(g0 + k * kWaves, g_end - 1) * kPanelRows];
-        }
-        int cs[kUnroll];
-#pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
-            const uint32_t w[8] = { q[k][0].x, q[k][0].y, q[k][0].z, q[k][0].w, q[k][1].x, q[k][1].y, q[k][1].z, q[k][1].w };
-            int c = 0;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) c = dot8(w[i], 0x11111111u, c);
-            cs[k] = c;
-        }
-#pragma unroll
-        for (int j = 0; j < kPairs; ++j) {
-            if (j + kRing - 1 < kPairs) fetch_pair(j + kRing - 1);
-            const int t = j / kUnroll, k = j % kUnroll, slot = j % kRing;
-            const uint32_t w[8] = { q[k][0].x, q[k][0].y, q[k][0].z, q[k][0].w, q[k][1].x, q[k][1].y, q[k][1].z, q[k][1].w };
+        for (int t = 0; t < T; ++t) {
+            const uint4 a0 = *reinterpret_cast<const uint4 *>(act + (gl * T + t) * 8);      // same address in every lane
+            const uint4 a1 = *reinterpret_cast<const uint4 *>(act + (gl * T + t) * 8 + 4);
             int acc = 0;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc = dot8(w[i], a[slot][i], acc);
-            const int mult = mzv[slot] & 0xFF;
-            const int zc = (int) (int8_t) ((mzv[slot] >> 8) & 0xFF);
-            int term = mult * (acc + zc * cs[k]);
-            if (hask) term *= kw[k];
-            if (g0 + k * kWaves < g_end) tot[t] += term >> kTermShift;
+            acc = dot8(w[0], a0.x, acc);
+            acc = dot8(w[1], a0.y, acc);
+            acc = dot8(w[2], a0.z, acc);
+            acc = dot8(w[3], a0.w, acc);
+            acc = dot8(w[4], a1.x, acc);
+            acc = dot8(w[5], a1.y, acc);
+            acc = dot8(w[6], a1.z, acc);
+            acc = dot8(w[7], a1.w, acc);
+            const int32_t mzv = mz[gl * T + t];
+            const int mult = mzv & 0xFF;
+            const int zc = (int) (int8_t) ((mzv >> 8) & 0xFF);
+            int term = mult * (acc + zc * cs);
+            if (hask) term *= kw;
+            tot[t] += term >> kTermShift;
         }
     }
 }
@@ -97,10 +95,15 @@ __device__ __forceinline__ void gemv_body(const uint4 *__restrict__ codes, const
 template <int T, int kWaves>
 __global__ void __launch_bounds__(kWaves * 64)
 rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
-               const int32_t *__restrict__ flags, const uint32_t *__restrict__ act, const int32_t *__restrict__ mz,
-               const float *__restrict__ u, float *__restrict__ y, int64_t ldy, int64_t N, int ng,
+               const int32_t *__restrict__ flags, const float *__restrict__ x, int64_t ldx,
+               const float *__restrict__ lohi, const float *__restrict__ rpart, float *__restrict__ y, int64_t ldy, int64_t N, int ng,
                unsigned long long *__restrict__ cells, int n_rows_pad) {
+    constexpr int NT = kWaves * 64;
     __shared__ int32_t red[kWaves][T][64];
+    __shared__ float s_R[T], s_u[T];
+    __shared__ float s_inv[kMaxSlice * T], s_zf[kMaxSlice * T];
+    __shared__ uint32_t s_act[kMaxSlice * T * 8];
+    __shared__ int32_t s_mz[kMaxSlice * T];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -108,18 +111,99 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     const int panel = blockIdx.x;
     const int nks = gridDim.y, ks = blockIdx.y;
     const int g_begin = (int) ((int64_t) ng * ks / nks), g_end = (int) ((int64_t) ng * (ks + 1) / nks);
+    const int cnt = g_end - g_begin;
 
+    // weights of the first batch go in flight before anything else
+    const uint4 *wp = codes + (size_t) panel * ng * 128 + lane;
+    const uint8_t *kp = kmul + (size_t) panel * ng * kPanelRows + lane;
+    Batch b0;
+    load_batch<kWaves>(b0, wp, g_begin + wave, g_end);
+
+    // The three inputs of the quantizer prologue do not depend on each other: fetch this thread's share of all of
+    // them now (partial range maxima, its first (group, token) range, its first code word's eight values), so the
+    // prologue pays one memory latency, not three in a row.
+    const int n_gt = cnt * T, n_words = n_gt * 8;
+    float pre_r = 0.0f;
+    if (tid < T * 64 && lane < kRangeParts) pre_r = rpart[(tid >> 6) * kRangeParts + lane];
+    float2 pre_lh = make_float2(0.0f, 0.0f);
+    if (tid < n_gt) pre_lh = reinterpret_cast<const float2 *>(lohi)[(size_t) (tid % T) * ng + g_begin + tid / T];
+    float4 pre_x0 = make_float4(0.f, 0.f, 0.f, 0.f), pre_x1 = pre_x0;
+    if (tid < n_words) {
+        const int gt = tid >> 3;
+        const float4 *xp = reinterpret_cast<const float4 *>(x + (int64_t) (gt % T) * ldx +
+                                                            (int64_t) (g_begin + gt / T) * kGroup + (tid & 7) * 8);
+        pre_x0 = xp[0];
+        pre_x1 = xp[1];
+    }
+
+    // ---- token units: R = widest clipped group range of the whole token (the activation kernel left 32 partial
+    // maxima per token), 2 if the token is all zero; u = R / 3825
+    if (tid < T * 64) {
+        for (int tt = tid >> 6; tt < T; tt += kWaves) {   // wavefront w handles tokens w, w + kWaves, ...
+            float r = tt == (tid >> 6) ? pre_r : (lane < kRangeParts ? rpart[tt * kRangeParts + lane] : 0.0f);
+            r = wave_max(r);
+            if (r == 0.0f) r = 2.0f;
+            if (lane == 0) {
+                s_R[tt] = r;
+                s_u[tt] = r / 3825.0f;  // 15 * 255
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- per (group of the slice, token): multiplier, 1 / (m u), zero point (reference lines 2662-2665)
+    for (int gt = tid; gt < n_gt; gt += NT) {
+        const int t = gt % T, g = g_begin + gt / T;
+        const float2 r = gt == tid ? pre_lh : reinterpret_cast<const float2 *>(lohi)[(size_t) t * ng + g];
+        const float lo = r.x, hi = r.y;
+        const int mg = (int) fminf(fmaxf(ceilf(((hi - lo) * 255.0f) / s_R[t]), 1.0f), 255.0f);
+        const float inv = 1.0f / ((float) mg * s_u[t]);
+        const float zf = fminf(fmaxf(rintf(-lo * inv), 0.0f), 15.0f);
+        s_inv[gt] = inv;
+        s_zf[gt] = zf;
+        s_mz[gt] = mg | ((8 - (int) zf) & 0xFF) << 8;
+    }
+    __syncthreads();
+
+    // ---- codes: a thread per code word (8 values), q = clamp(rint(x * inv) + z, 0, 15) (lines 2670-2675)
+    for (int id = tid; id < n_words; id += NT) {
+        const int wi = id & 7, gt = id >> 3;
+        const int t = gt % T, g = g_begin + gt / T;
+        const float inv = s_inv[gt], zf = s_zf[gt];
+        float4 v0 = pre_x0, v1 = pre_x1;
+        if (id != tid) {
+            const float4 *xp = reinterpret_cast<const float4 *>(x + (int64_t) t * ldx + (int64_t) g * kGroup + wi * 8);
+            v0 = xp[0];
+            v1 = xp[1];
+        }
+        const float f[8] = { v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w };
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int q = (int) fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
+            word |= (uint32_t) ((q - 8) & 0xF) << (4 * j);
+        }
+        s_act[id] = word;
+    }
+    __syncthreads();
+
+    // ---- the product
+    const bool hask = *reinterpret_cast<const volatile int32_t *>(flags) & 1;
     int32_t tot[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) tot[t] = 0;
-
-    gemv_body<T, kWaves>(codes, kmul, act, mz, flags, panel, ng, g_begin, g_end, wave, lane, tot);
+    compute_batch<T, kWaves>(b0, kp, hask, s_act, s_mz, g_begin + wave, g_begin, g_end, tot);
+    for (int g0 = g_begin + wave + kWaves * kUnroll; g0 < g_end; g0 += kWaves * kUnroll) {
+        Batch b;
+        load_batch<kWaves>(b, wp, g0, g_end);
+        compute_batch<T, kWaves>(b, kp, hask, s_act, s_mz, g0, g_begin, g_end, tot);
+    }
 
 #pragma unroll
     for (int t = 0; t < T; ++t) red[wave][t][lane] = tot[t];
     __syncthreads();
 
-    for (int item = tid; item < T * 64; item += kWaves * 64) {
+    for (int item = tid; item < T * 64; item += NT) {
         const int t = item >> 6;
         const int64_t n = (int64_t) panel * kPanelRows + lane;
         int32_t sum = 0;
@@ -139,7 +223,7 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
             __hip_atomic_store(cell, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             sum = (int32_t) (uint32_t) now;  // the total fits int32 by construction of the format
         }
-        if (n < N) y[(int64_t) t * ldy + n] = (((float) sum * 16.0f) * u[t]) * s_w[n];
+        if (n < N) y[(int64_t) t * ldy + n] = (((float) sum * 16.0f) * s_u[t]) * s_w[n];
     }
 }
 
@@ -149,7 +233,7 @@ hipError_t launch_tw(const GemvArgs &a, int nks, hipStream_t stream) {
     hipLaunchKernelGGL((rq_gemv_kernel<T, kWaves>), dim3(a.L.n_panels, nks), dim3(kWaves * 64), 0, stream,
                        reinterpret_cast<const uint4 *>(p + a.L.off_codes),
                        reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,
-                       reinterpret_cast<const int32_t *>(p + a.L.off_flags), a.act, a.mz, a.u, a.y, a.ldy, a.L.N,
+                       reinterpret_cast<const int32_t *>(p + a.L.off_flags), a.x, a.ldx, a.lohi, a.rpart, a.y, a.ldy, a.L.N,
                        a.L.ng, reinterpret_cast<unsigned long long *>(a.tot), a.L.n_panels * kPanelRows);
     return hipGetLastError();
 }
@@ -168,8 +252,8 @@ hipError_t launch_t(const GemvArgs &a, int nks, hipStream_t stream) {
 
 // How many workgroups share K for one panel. The kernel is a pure stream with a latency-bound start and end, so
 // it wants many small workgroups: their starts and tails overlap and the last wave of workgroups is short. Aim for
-// about a thousand workgroups, at least a batch (kGemvWaves x kUnroll groups) each when K allows, and never fewer
-// than four groups per workgroup.
+// about a thousand workgroups, at least a batch (kGemvWaves x kUnroll groups) each when K allows, never fewer than
+// four groups per workgroup, and never more than kMaxSlice (the slice's codes live in LDS).
 int gemv_ksplit(const PreparedLayout &L) {
     static const int forced = getenv("RQ_GEMV_KSPLIT") ? atoi(getenv("RQ_GEMV_KSPLIT")) : 0;
     int nks;
@@ -181,6 +265,8 @@ int gemv_ksplit(const PreparedLayout &L) {
         nks = by_batch > by_grid ? by_batch : by_grid;
         if (nks > L.ng / 4) nks = L.ng / 4;
     }
+    const int least = (L.ng + kMaxSlice - 1) / kMaxSlice;   // ceil(ng / nks) <= kMaxSlice
+    if (nks < least) nks = least;
     if (nks > L.ng) nks = L.ng;
     return nks < 1 ? 1 : nks;
 }

@@ -1,0 +1,142 @@
+// Building blocks of the online Hadamard shared by the activation kernels: the Paley sign table and its unrolled
+// column sums, the register butterflies of the Sylvester transform, the padded LDS row.
+#pragma once
+
+#include "rq_common.h"
+
+#pragma clang fp contract(off)
+
+namespace rq {
+namespace had {
+
+// ---- Paley construction I, as signs: neg[i][a] is true where A[i][a] = -1 (reference lines 2433-2448) ----
+template <int P>
+struct PaleyTable {
+    bool neg[P][P];
+};
+
+template <int P>
+constexpr PaleyTable<P> make_paley() {
+    PaleyTable<P> t{};
+    constexpr int q = P - 1;
+    bool residue[P] = {};
+    for (int r = 1; r < q; ++r) residue[(r * r) % q] = true;
+    for (int i = 0; i < P; ++i) {
+        for (int a = 0; a < P; ++a) {
+            bool n = false;
+            if (i == a || i == 0) {
+                n = false;                       // diagonal and first row are +1
+            } else if (a == 0) {
+                n = true;                        // first column below the diagonal is -1
+            } else {
+                n = !residue[(((a - i) % q) + q) % q];
+            }
+            t.neg[i][a] = n;
+        }
+    }
+    return t;
+}
+
+// outputs 4S .. 4S+3 of one column: acc = ((0 +- c0) +- c1) ... in ascending chunk order
+template <int P, int S>
+__device__ __forceinline__ void paley_slice(const float (&col)[P], float (&out)[4]) {
+    constexpr PaleyTable<P> T = make_paley<P>();
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < P; ++i) {
+            acc = T.neg[i][4 * S + o] ? acc - col[i] : acc + col[i];
+        }
+        out[o] = acc;
+    }
+}
+
+template <int P, int S = 0>
+__device__ __forceinline__ void paley_pick(int s, const float (&col)[P], float (&out)[4]) {
+    if (s == S) {
+        paley_slice<P, S>(col, out);
+    } else if constexpr (S + 1 < P / 4) {
+        paley_pick<P, S + 1>(s, col, out);
+    }
+}
+
+// all P outputs of one column, written back in place (the column is private to the calling thread)
+template <int P, int S = 0>
+__device__ __forceinline__ void paley_column(const float (&col)[P], float *dst, int stride, float scale) {
+    float out[4];
+    paley_slice<P, S>(col, out);
+#pragma unroll
+    for (int o = 0; o < 4; ++o) dst[(4 * S + o) * stride] = out[o] * scale;
+    if constexpr (S + 1 < P / 4) paley_column<P, S + 1>(col, dst, stride, scale);
+}
+
+// same, for chunk lengths that are not a multiple of 16 (the padded stride is then not uniform)
+template <int P, int S = 0>
+__device__ __forceinline__ void paley_column_generic(const float (&col)[P], float *buf, int b0, int m, float scale) {
+    float out[4];
+    paley_slice<P, S>(col, out);
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+        const int i = b0 + (4 * S + o) * m;
+        buf[i + (i >> 4)] = out[o] * scale;
+    }
+    if constexpr (S + 1 < P / 4) paley_column_generic<P, S + 1>(col, buf, b0, m, scale);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// The row sits in LDS with one float of padding after every 16: element i lives at i + i / 16. With it the
+// strided accesses of the register butterflies (16 elements 16, 256, ... apart) spread over all banks.
+__device__ __forceinline__ int padi(int i) { return i + (i >> 4); }
+
+// One pass of the Sylvester transform: R = 2^LR elements `1 << ls` apart go through LR butterfly stages in
+// registers (strides 1 << ls, 2 << ls, ...; lower index gets a + b, upper a - b, as reference lines 2454-2464).
+// Successive passes run in ascending stride order, so every element sees the reference's stage order.
+template <int LR>
+__device__ __forceinline__ void fwht_pass(float *buf, int K, int lm, int ls, int tid, int nt) {
+    constexpr int R = 1 << LR;
+    const int units = K >> LR;
+    for (int u = tid; u < units; u += nt) {
+        const int c = u >> (lm - LR), ul = u & ((1 << (lm - LR)) - 1);
+        const int low = ul & ((1 << ls) - 1), high = ul >> ls;
+        const int base = (c << lm) + ((high << (ls + LR)) | low);
+        float v[R];
+#pragma unroll
+        for (int j = 0; j < R; ++j) v[j] = buf[padi(base + (j << ls))];
+#pragma unroll
+        for (int h = 1; h < R; h <<= 1) {
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                if ((j & h) == 0) {
+                    const float lo = v[j], up = v[j + h];
+                    v[j] = lo + up;
+                    v[j + h] = lo - up;
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < R; ++j) buf[padi(base + (j << ls))] = v[j];
+    }
+}
+
+
+// all Sylvester stages of every chunk of m = 1 << lm floats of a padded row, four stages per trip through LDS
+__device__ __forceinline__ void fwht_row(float *buf, int K, int lm, int tid, int nt) {
+    for (int ls = 0; ls < lm;) {
+        const int lr = lm - ls < 4 ? lm - ls : 4;
+        if (lr == 4) fwht_pass<4>(buf, K, lm, ls, tid, nt);
+        else if (lr == 3) fwht_pass<3>(buf, K, lm, ls, tid, nt);
+        else if (lr == 2) fwht_pass<2>(buf, K, lm, ls, tid, nt);
+        else fwht_pass<1>(buf, K, lm, ls, tid, nt);
+        ls += lr;
+        __syncthreads();
+    }
+}
+
+}  // namespace had
+}  // namespace rq

@@ -5,12 +5,13 @@
 //
 // Bit-exactness with the CPU reference (ggml_rq_hadamard, reference patch lines 2450-2485, and
 // rq_quantize_row_a, lines 2639-2679) rests on three rules that this file keeps:
-//   * Sylvester stages are exact pairs (a + b, a - b), stride ascending; which lane computes a pair is free.
+//   * Sylvester stages are exact pairs (a + b, a - b), stride ascending; which lane computes a pair is free, so
+//     four stages at a time run in registers (16 elements per thread) between two trips through LDS.
 //   * The Paley stage adds the p chunk values of a column strictly in ascending chunk order, starting from
 //     +0.0f, one rounding per add; the signs are compile-time constants so each term is one v_add / v_sub.
 //   * Every product, sum and quotient of the quantizer is a separate correctly rounded fp32 operation
 //     (no contraction, IEEE division, denormals kept).
-#include "rq_common.h"
+#include "rq_hadamard.h"
 
 #pragma clang fp contract(off)
 
@@ -20,73 +21,7 @@ namespace {
 
 constexpr int kNT = 512;  // threads per token workgroup
 
-// ---- Paley construction I, as signs: neg[i][a] is true where A[i][a] = -1 (reference lines 2433-2448) ----
-template <int P>
-struct PaleyTable {
-    bool neg[P][P];
-};
-
-template <int P>
-constexpr PaleyTable<P> make_paley() {
-    PaleyTable<P> t{};
-    constexpr int q = P - 1;
-    bool residue[P] = {};
-    for (int r = 1; r < q; ++r) residue[(r * r) % q] = true;
-    for (int i = 0; i < P; ++i) {
-        for (int a = 0; a < P; ++a) {
-            bool n = false;
-            if (i == a || i == 0) {
-                n = false;                       // diagonal and first row are +1
-            } else if (a == 0) {
-                n = true;                        // first column below the diagonal is -1
-            } else {
-                n = !residue[(((a - i) % q) + q) % q];
-            }
-            t.neg[i][a] = n;
-        }
-    }
-    return t;
-}
-
-// outputs 4S .. 4S+3 of one column: acc = ((0 +- c0) +- c1) ... in ascending chunk order
-template <int P, int S>
-__device__ __forceinline__ void paley_slice(const float (&col)[P], float (&out)[4]) {
-    constexpr PaleyTable<P> T = make_paley<P>();
-#pragma unroll
-    for (int o = 0; o < 4; ++o) {
-        float acc = 0.0f;
-#pragma unroll
-        for (int i = 0; i < P; ++i) {
-            acc = T.neg[i][4 * S + o] ? acc - col[i] : acc + col[i];
-        }
-        out[o] = acc;
-    }
-}
-
-template <int P, int S = 0>
-__device__ __forceinline__ void paley_pick(int s, const float (&col)[P], float (&out)[4]) {
-    if (s == S) {
-        paley_slice<P, S>(col, out);
-    } else if constexpr (S + 1 < P / 4) {
-        paley_pick<P, S + 1>(s, col, out);
-    }
-}
-
-// all P outputs of one column, written back in place (the column is private to the calling thread)
-template <int P, int S = 0>
-__device__ __forceinline__ void paley_column(const float (&col)[P], float *dst, int stride, float scale) {
-    float out[4];
-    paley_slice<P, S>(col, out);
-#pragma unroll
-    for (int o = 0; o < 4; ++o) dst[(4 * S + o) * stride] = out[o] * scale;
-    if constexpr (S + 1 < P / 4) paley_column<P, S + 1>(col, dst, stride, scale);
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
-}
+using namespace had;
 
 template <int P, bool SLICED>
 __global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs a) {
@@ -95,7 +30,7 @@ __global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs
 
     const int tid = threadIdx.x;
     if ((int) blockIdx.x >= a.token_blocks) {
-        // blocks past the tokens clear the split-K sums and arrival counters of the product kernel
+        // blocks past the tokens clear the split-K cells of the product kernel
         const int64_t i0 = ((int64_t) (blockIdx.x - a.token_blocks) * kNT + tid) * 4;
         if (i0 + 3 < a.zero_ints) {
             *reinterpret_cast<int4 *>(a.zero_ptr + i0) = make_int4(0, 0, 0, 0);
@@ -108,67 +43,82 @@ __global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs
     const int t = blockIdx.x;
     const int K = a.K;
     const int ng = K / kGroup;
+    const int Kp = padi(K) + 1;                  // floats of one padded row
     float *buf = smem;
-    float *alt = smem + K;                       // second row buffer (SLICED only)
-    float *g_lo = smem + (SLICED ? 2 * K : K);
+    float *alt = smem + Kp;                      // second row buffer (SLICED only)
+    float *g_lo = smem + (SLICED ? 2 * Kp : Kp);
     float *g_hi = g_lo + ng;
 
     const float *xr = a.x + (int64_t) t * a.ldx;
     for (int i = tid * 4; i < K; i += kNT * 4) {
-        *reinterpret_cast<float4 *>(buf + i) = *reinterpret_cast<const float4 *>(xr + i);
+        const float4 v = *reinterpret_cast<const float4 *>(xr + i);
+        float *d = buf + padi(i);                // i % 4 == 0: the four land in one run of 16
+        d[0] = v.x;
+        d[1] = v.y;
+        d[2] = v.z;
+        d[3] = v.w;
     }
     __syncthreads();
 
     if (a.rotate) {
         const int m = a.m;
-        // Sylvester butterflies inside every chunk of m, stride 1, 2, 4, ... (reference lines 2454-2464)
-        if (m > 1) {
-            const int half = m >> 1;
-            const int lhalf = __ffs(half) - 1;
-            for (int h = 1; h < m; h <<= 1) {
-                for (int q = tid; q < (K >> 1); q += kNT) {
-                    const int c = q >> lhalf, r = q & (half - 1);
-                    const int j = ((r & ~(h - 1)) << 1) | (r & (h - 1));
-                    float *v = buf + c * m + j;
-                    const float lo = v[0], up = v[h];
-                    v[0] = lo + up;
-                    v[h] = lo - up;
-                }
-                __syncthreads();
-            }
-        }
+        const int lm = __ffs(m) - 1;
+        fwht_row(buf, K, lm, tid, kNT);
         if constexpr (P > 1) {
             // Paley across the P chunks of every rotation block (reference lines 2466-2482), then the scale
             const int ncols = K / P;  // columns of all rotation blocks of this token
+            const bool m16 = (m & 15) == 0;
+            const int pm = m + (m >> 4);
             if constexpr (SLICED) {
-                for (int id = tid; id < (K >> 2); id += kNT) {
-                    const int s = id / ncols, cidx = id - s * ncols;
+                // wave-items = (slice of four outputs, run of 64 columns); each wavefront takes a contiguous block
+                // of them, so it stays in one slice's straight-line code for several items in a row
+                const int col_runs = (ncols + 63) >> 6;
+                const int n_items = (P / 4) * col_runs;
+                const int per_wave = (n_items + kNT / 64 - 1) / (kNT / 64);
+                const int wave = tid >> 6, lane = tid & 63;
+                for (int it = 0; it < per_wave; ++it) {
+                    const int wi = wave * per_wave + it;
+                    if (wi >= n_items) break;
+                    const int s = wi / col_runs, cidx = (wi - s * col_runs) * 64 + lane;
+                    if (cidx >= ncols) continue;
                     const int rb = cidx / m, j = cidx - rb * m;
-                    const float *src = buf + rb * a.n_rot + j;
+                    const int b0 = rb * a.n_rot + j;
                     float col[P];
+                    if (m16) {
+                        const float *src = buf + padi(b0);
 #pragma unroll
-                    for (int i = 0; i < P; ++i) col[i] = src[i * m];
+                        for (int i = 0; i < P; ++i) col[i] = src[i * pm];
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < P; ++i) col[i] = buf[padi(b0 + i * m)];
+                    }
                     float out[4];
                     paley_pick<P>(s, col, out);
-                    float *dst = alt + rb * a.n_rot + j + 4 * s * m;
 #pragma unroll
-                    for (int o = 0; o < 4; ++o) dst[o * m] = out[o] * a.scale;
+                    for (int o = 0; o < 4; ++o) alt[padi(b0 + (4 * s + o) * m)] = out[o] * a.scale;
                 }
                 __syncthreads();
                 float *tmp = buf; buf = alt; alt = tmp;
             } else {
                 for (int cidx = tid; cidx < ncols; cidx += kNT) {
                     const int rb = cidx / m, j = cidx - rb * m;
-                    float *src = buf + rb * a.n_rot + j;
+                    const int b0 = rb * a.n_rot + j;
                     float col[P];
+                    if (m16) {
+                        float *src = buf + padi(b0);
 #pragma unroll
-                    for (int i = 0; i < P; ++i) col[i] = src[i * m];
-                    paley_column<P>(col, src, m, a.scale);
+                        for (int i = 0; i < P; ++i) col[i] = src[i * pm];
+                        paley_column<P>(col, src, pm, a.scale);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < P; ++i) col[i] = buf[padi(b0 + i * m)];
+                        paley_column_generic<P>(col, buf, b0, m, a.scale);
+                    }
                 }
                 __syncthreads();
             }
         } else {
-            for (int i = tid; i < K; i += kNT) buf[i] = buf[i] * a.scale;
+            for (int i = tid; i < K; i += kNT) buf[padi(i)] = buf[padi(i)] * a.scale;
             __syncthreads();
         }
     }
@@ -176,7 +126,8 @@ __global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs
     if (a.mode == kActRotateOnly) {
         float *o = a.out_f32 + (int64_t) t * a.ldo;
         for (int i = tid * 4; i < K; i += kNT * 4) {
-            *reinterpret_cast<float4 *>(o + i) = *reinterpret_cast<const float4 *>(buf + i);
+            const float *sp = buf + padi(i);
+            *reinterpret_cast<float4 *>(o + i) = make_float4(sp[0], sp[1], sp[2], sp[3]);
         }
         return;
     }
@@ -189,8 +140,9 @@ __global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs
         const bool on = w < nw;
         float mn = 0.0f, mx = 0.0f;
         if (on) {
-            const float4 v0 = *reinterpret_cast<const float4 *>(buf + 8 * w);
-            const float4 v1 = *reinterpret_cast<const float4 *>(buf + 8 * w + 4);
+            const float *sp = buf + padi(8 * w);   // 8 consecutive values never straddle a run of 16
+            const float4 v0 = make_float4(sp[0], sp[1], sp[2], sp[3]);
+            const float4 v1 = make_float4(sp[4], sp[5], sp[6], sp[7]);
             mn = fminf(fminf(fminf(fminf(mn, v0.x), fminf(v0.y, v0.z)), fminf(fminf(v0.w, v1.x), fminf(v1.y, v1.z))), v1.w);
             mx = fmaxf(fmaxf(fmaxf(fmaxf(mx, v0.x), fmaxf(v0.y, v0.z)), fmaxf(fmaxf(v0.w, v1.x), fmaxf(v1.y, v1.z))), v1.w);
         }
@@ -207,6 +159,25 @@ __global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs
             }
             rmax = fmaxf(rmax, hi - lo);
         }
+    }
+    if (a.mode == kActStats) {
+        rmax = wave_max(rmax);
+        if ((tid & 63) == 0) a.rpart[(size_t) t * kRangeParts + (tid >> 6)] = rmax;
+        if (tid >= kNT / 64 && tid < kRangeParts) a.rpart[(size_t) t * kRangeParts + tid] = 0.0f;
+        __syncthreads();
+        float *lh = a.lohi + (size_t) t * ng * 2;
+        for (int g = tid; g < ng; g += kNT) {
+            lh[2 * g] = g_lo[g];
+            lh[2 * g + 1] = g_hi[g];
+        }
+        if (a.out_f32 != nullptr) {
+            float *o = a.out_f32 + (int64_t) t * a.ldo;
+            for (int i = tid * 4; i < K; i += kNT * 4) {
+                const float *sp = buf + padi(i);
+                *reinterpret_cast<float4 *>(o + i) = make_float4(sp[0], sp[1], sp[2], sp[3]);
+            }
+        }
+        return;
     }
     rmax = wave_max(rmax);
     if ((tid & 63) == 0) s_red[tid >> 6] = rmax;
@@ -229,9 +200,8 @@ __global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs
         const float inv = 1.0f / ((float) mg * u);
         const float zf = fminf(fmaxf(rintf(-lo * inv), 0.0f), 15.0f);
         const int z = (int) zf;
-        const float4 v0 = *reinterpret_cast<const float4 *>(buf + 8 * wc);
-        const float4 v1 = *reinterpret_cast<const float4 *>(buf + 8 * wc + 4);
-        const float f[8] = { v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w };
+        const float *sp = buf + padi(8 * wc);
+        const float f[8] = { sp[0], sp[1], sp[2], sp[3], sp[4], sp[5], sp[6], sp[7] };
         int q[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) q[j] = (int) fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
@@ -268,14 +238,7 @@ __global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs
 #pragma unroll
         for (int j = 0; j < 8; ++j) word |= (uint32_t) ((q[j] - 8) & 0xF) << (4 * j);
 
-        if (a.mode == kActQ4) {
-            if (on) {
-                const int chunk = t >> 3, slot = t & 7;
-                const size_t cell = ((size_t) chunk * ng + g) * kGemvTokens + slot;
-                a.act[cell * 8 + (w & 7)] = word;
-                if ((tid & 7) == 0) reinterpret_cast<int32_t *>(a.mz)[cell] = mg | ((8 - z) & 0xFF) << 8;
-            }
-        } else {  // kActBlocks: the reference's A4 / A4H storage (reference lines 2656-2661, 2667-2669)
+        {  // kActBlocks: the reference's A4 / A4H storage (reference lines 2656-2661, 2667-2669)
             const int base = tid & 32;  // lanes base, base+8, base+16, base+24 hold the block's four groups
             uint32_t zs = 0, ms = 0;
 #pragma unroll
@@ -310,14 +273,16 @@ hipError_t launch_one(const RotQuantArgs &a, size_t lds, int grid, hipStream_t s
     return hipGetLastError();
 }
 
+// LDS: one padded row (two when the Paley stage is sliced over more threads) plus the group ranges. Slicing buys
+// parallelism inside a token and costs occupancy, so it is for small batches only.
 template <int P>
 hipError_t launch_p(const RotQuantArgs &a, int grid, hipStream_t stream) {
-    const size_t stats = (size_t) 2 * (a.K / kGroup) * sizeof(float);
-    const size_t lds_sliced = (size_t) 2 * a.K * sizeof(float) + stats;
-    if (P > 1 && lds_sliced <= 160 * 1024 - 64) {
-        return launch_one<P, (P > 1)>(a, lds_sliced, grid, stream);
+    const size_t row = (size_t) (a.K + (a.K >> 4) + 1) * sizeof(float);
+    const size_t stats = (size_t) 2 * (a.K / kGroup + 1) * sizeof(float);
+    if (P > 1 && a.M <= 64 && 2 * row + stats <= 160 * 1024 - 64) {
+        return launch_one<P, (P > 1)>(a, 2 * row + stats, grid, stream);
     }
-    return launch_one<P, false>(a, (size_t) a.K * sizeof(float) + stats, grid, stream);
+    return launch_one<P, false>(a, row + stats, grid, stream);
 }
 
 }  // namespace
