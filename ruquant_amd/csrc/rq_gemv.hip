@@ -113,14 +113,8 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     const int g_begin = (int) ((int64_t) ng * ks / nks), g_end = (int) ((int64_t) ng * (ks + 1) / nks);
     const int cnt = g_end - g_begin;
 
-    // weights of the first batch go in flight before anything else
-    const uint4 *wp = codes + (size_t) panel * ng * 128 + lane;
-    const uint8_t *kp = kmul + (size_t) panel * ng * kPanelRows + lane;
-    Batch b0;
-    load_batch<kWaves>(b0, wp, g_begin + wave, g_end);
-
     // The three inputs of the quantizer prologue do not depend on each other: fetch this thread's share of all of
-    // them now (partial range maxima, its first (group, token) range, its first code word's eight values), so the
+    // them first (partial range maxima, its first (group, token) range, its first code word's eight values), so the
     // prologue pays one memory latency, not three in a row.
     const int n_gt = cnt * T, n_words = n_gt * 8;
     float pre_r = 0.0f;
@@ -135,6 +129,13 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
         pre_x0 = xp[0];
         pre_x1 = xp[1];
     }
+
+    // ... and right behind them the weights of the first batch. This order matters: a wavefront's loads complete in
+    // issue order, so the small prologue inputs must be the OLDER loads or they would wait for 10 KiB of weights.
+    const uint4 *wp = codes + (size_t) panel * ng * 128 + lane;
+    const uint8_t *kp = kmul + (size_t) panel * ng * kPanelRows + lane;
+    Batch b0;
+    load_batch<kWaves>(b0, wp, g_begin + wave, g_end);
 
     // ---- token units: R = widest clipped group range of the whole token (the activation kernel left 32 partial
     // maxima per token), 2 if the token is all zero; u = R / 3825
