@@ -39,7 +39,8 @@ namespace {
 struct Env {
     float clip[2];   // RQ_ACT_CLIP, RQ_ACT_CLIP_H (falls back to the former); -1 = unset
     int   act_group;
-    int   gemm_min;  // smallest token count that takes the MFMA GEMM
+    int   gemm_min;  // smallest token count that takes the tiled MFMA GEMM
+    int   gemv_max;  // largest token count that takes the GEMV; between the two: the skinny MFMA kernel
     Env() {
         const char *e = getenv("RQ_ACT_CLIP");
         const char *eh = getenv("RQ_ACT_CLIP_H");
@@ -49,9 +50,13 @@ struct Env {
         const int v = g ? atoi(g) : 64;
         act_group = v == 128 || v == 256 ? v : 64;
         const char *gm = getenv("RQ_GEMM_MIN");
-        gemm_min = gm ? atoi(gm) : 33;
+        gemm_min = gm ? atoi(gm) : kSkinnyTokens + 1;
         if (gemm_min < 1) gemm_min = 1;
-        if (gemm_min > kGemvMaxTokens + 1) gemm_min = kGemvMaxTokens + 1;
+        if (gemm_min > kSkinnyTokens + 1) gemm_min = kSkinnyTokens + 1;
+        const char *gv = getenv("RQ_GEMV_MAX");
+        gemv_max = gv ? atoi(gv) : kGemvTokens;
+        if (gemv_max < 0) gemv_max = 0;
+        if (gemv_max > kGemvMaxTokens) gemv_max = kGemvMaxTokens;
     }
 };
 
@@ -79,7 +84,11 @@ bool rotation_of(int type, int64_t K, int64_t n_rot, int &p, int &m) {
     return hadamard_factor(n_rot, p, m);
 }
 
-bool use_gemm(int64_t M) { return M >= env().gemm_min; }
+enum Path { kPathGemv, kPathSkinny, kPathGemm };
+Path path_of(int64_t M) {
+    if (M >= env().gemm_min) return kPathGemm;
+    return M <= env().gemv_max ? kPathGemv : kPathSkinny;
+}
 
 int run_products(int type, int n, const void *const *prepared, int64_t K, const int64_t *N, const float *x,
                  int64_t ldx, int64_t M, float *const *y, const int64_t *ldy, float clip, int64_t n_rot, void *ws,
@@ -103,7 +112,8 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     if (ws_bytes < W.bytes || (reinterpret_cast<uintptr_t>(ws) & 255) != 0) return RQ_E_WORKSPACE;
     uint8_t *wsb = reinterpret_cast<uint8_t *>(ws);
 
-    const bool gemm = use_gemm(M);
+    const Path path = path_of(M);
+    const bool gemm = path != kPathGemv;   // the int8 digit planes feed both MFMA kernels
     RotQuantArgs q;
     memset(&q, 0, sizeof q);
     q.x = x;
@@ -119,7 +129,10 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     q.mode = gemm ? kActI8 : kActStats;
     q.u = reinterpret_cast<float *>(wsb + W.off_u);
     q.act = reinterpret_cast<uint32_t *>(wsb + W.off_act);
-    q.Mp = (int) W.Mp;
+    // token stride of the digit planes: the GEMM pads to its tile; the skinny kernel wants them dense (a padded
+    // plane would put all of its reads on the few L2 channels that the used 256 bytes of every 2 KB map to)
+    const int act_mp = path == kPathSkinny ? (int) ((M + 15) / 16 * 16) : (int) W.Mp;
+    q.Mp = act_mp;
     const float *gemv_x = x;      // what the GEMV quantizes from: the rotated rows, or x itself for W4A4
     int64_t gemv_ldx = ldx;
     if (!gemm) {
@@ -135,6 +148,9 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
         // only the token slots this call can touch: [min(M, 8)][padded rows] cells of two ints
         const int64_t slots = M < kGemvTokens ? M : kGemvTokens;
         q.zero_ints = 2 * slots * (int64_t) ((Nmax + kPanelRows - 1) / kPanelRows * kPanelRows);
+    } else if (path == kPathSkinny) {
+        q.zero_ptr = reinterpret_cast<int32_t *>(wsb + W.off_tot);
+        q.zero_ints = 2 * M * (int64_t) ((Nmax + kPanelRows - 1) / kPanelRows * kPanelRows);
     }
     hipError_t e = hipSuccess;
     if (stages & 1) {
@@ -145,7 +161,20 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
 
     for (int i = 0; i < n; ++i) {
         const PreparedLayout L = prepared_layout(K, N[i]);
-        if (gemm) {
+        if (path == kPathSkinny) {
+            SkinnyArgs g;
+            g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
+            g.L = L;
+            g.act8 = wsb + W.off_act;
+            g.u = q.u;
+            g.y = y[i];
+            g.ldy = ldy[i];
+            g.M = (int) M;
+            g.Mp = act_mp;
+            g.tot = reinterpret_cast<int32_t *>(wsb + W.off_tot);
+            e = launch_skinny(g, stream);
+            if (e != hipSuccess) return (int) e;
+        } else if (gemm) {
             GemmArgs g;
             g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
             g.L = L;

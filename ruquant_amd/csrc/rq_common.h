@@ -15,6 +15,7 @@ constexpr int kTermShift  = 4;    // RQ_TERM_SHIFT (reference patch line 39)
 constexpr int kGemvTokens = 8;    // tokens per GEMV pass; the activation slot stride of the int4 layout
 constexpr int kGemmTokens = 128;  // token tile of the MFMA GEMM; int8 activations are padded to it
 constexpr int kRangeParts = 32;    // partial maxima of a token's group ranges handed from the activation kernel to the GEMV
+constexpr int kSkinnyTokens = 64;   // most tokens of one pass of the skinny MFMA kernel
 constexpr int kGemvMaxTokens = 64;  // the dispatcher never sends more tokens than this down the GEMV path
 
 // ---------------------------------------------------------------------------------------------------
@@ -66,7 +67,8 @@ inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
 //            the K slice it consumes itself.
 //            GEMM path: two int8 digit planes of m (q - z), [g][digit][quarter][Mp][16 bytes], in the byte order
 //            the weight unpack produces.
-//   cells  : split-K cells [8 tokens][n_panels * 64], 64 bits each: arrival count above bit 48, exact sum below.
+//   cells  : split-K cells [8 or 64 tokens][n_panels * 64], 64 bits each: arrival count above bit 48, exact sum
+//            below.
 // ---------------------------------------------------------------------------------------------------
 struct WorkspaceLayout {
     int64_t Mp;       // tokens padded to the GEMM tile
@@ -94,7 +96,7 @@ inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
     W.off_rpart = W.off_lohi + align_up(lohi, 256);
     const size_t gemv_form = align_up(rows, 256) + align_up(lohi, 256) + align_up(rpart, 256);
     off = align_up(off + (small && gemv_form > act_i8 ? gemv_form : act_i8), 256);
-    W.tot_ints = (size_t) 2 * kGemvTokens * n_panels * kPanelRows;
+    W.tot_ints = (size_t) 2 * (M <= kGemvTokens ? kGemvTokens : kSkinnyTokens) * n_panels * kPanelRows;
     W.off_tot = off;
     off = align_up(off + W.tot_ints * sizeof(int32_t), 256);
     W.bytes = off;
@@ -164,6 +166,20 @@ struct GemmArgs {
     int             M, Mp;
 };
 hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
+
+// 9..64 tokens: MFMA arithmetic on a GEMV-shaped weight stream; same operands as the GEMM plus the split-K cells
+struct SkinnyArgs {
+    const uint8_t  *prepared;
+    PreparedLayout  L;
+    const uint8_t  *act8;   // [g][digit][quarter][Mp][16]
+    const float    *u;      // [Mp]
+    float          *y;
+    int64_t         ldy;
+    int             M, Mp;
+    int32_t        *tot;    // split-K cells [M][n_panels * 64], 64 bits each
+};
+hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream);
+int skinny_ksplit(const PreparedLayout &L, int M);
 
 hipError_t launch_prepare(const void *blocks, const PreparedLayout &L, uint8_t *prepared, hipStream_t stream);
 

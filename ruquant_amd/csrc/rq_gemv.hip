@@ -97,7 +97,7 @@ __global__ void __launch_bounds__(kWaves * 64)
 rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                const int32_t *__restrict__ flags, const float *__restrict__ x, int64_t ldx,
                const float *__restrict__ lohi, const float *__restrict__ rpart, float *__restrict__ y, int64_t ldy, int64_t N, int ng,
-               unsigned long long *__restrict__ cells, int n_rows_pad) {
+               unsigned long long *__restrict__ cells, int n_rows_pad, int slice_base, int slice_extra) {
     constexpr int NT = kWaves * 64;
     __shared__ int32_t red[kWaves][T][64];
     __shared__ float s_R[T], s_u[T];
@@ -110,7 +110,9 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int panel = blockIdx.x;
     const int nks = gridDim.y, ks = blockIdx.y;
-    const int g_begin = (int) ((int64_t) ng * ks / nks), g_end = (int) ((int64_t) ng * (ks + 1) / nks);
+    // slices of ng / nks groups, the first ng % nks one longer (no division on the device)
+    const int g_begin = ks * slice_base + (ks < slice_extra ? ks : slice_extra);
+    const int g_end = g_begin + slice_base + (ks < slice_extra ? 1 : 0);
     const int cnt = g_end - g_begin;
 
     // The three inputs of the quantizer prologue do not depend on each other: fetch this thread's share of all of
@@ -235,7 +237,8 @@ hipError_t launch_tw(const GemvArgs &a, int nks, hipStream_t stream) {
                        reinterpret_cast<const uint4 *>(p + a.L.off_codes),
                        reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,
                        reinterpret_cast<const int32_t *>(p + a.L.off_flags), a.x, a.ldx, a.lohi, a.rpart, a.y, a.ldy, a.L.N,
-                       a.L.ng, reinterpret_cast<unsigned long long *>(a.tot), a.L.n_panels * kPanelRows);
+                       a.L.ng, reinterpret_cast<unsigned long long *>(a.tot), a.L.n_panels * kPanelRows, a.L.ng / nks,
+                       a.L.ng % nks);
     return hipGetLastError();
 }
 

@@ -143,6 +143,17 @@ def test_mul_mat_weight_multipliers(oracle, wgroup, M):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
+@pytest.mark.parametrize("M", [9, 15, 16, 31, 33, 47, 49, 63])
+def test_mul_mat_token_counts_between_gemv_and_gemm(oracle, M):
+    """Every fill of the 16-token tiles of the kernel that serves 9..64 tokens, with split K and a ragged N."""
+    N, K, type_ = 1000, 5120, rq.TYPE_W4A4H
+    blocks, wf, W = _weights(oracle, N, K, type_)
+    x = adversarial_activations(M, K, type_, wf, seed=M)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=K)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
 def test_mul_mat_block_diagonal_rotation(oracle):
     """Hadamard length shorter than the row (pad[0] = K / 4), as ruquant convert --rot-blocks writes."""
     N, K, M, type_ = 128, 6144, 9, rq.TYPE_W4A4H
