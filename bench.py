@@ -24,6 +24,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+# HBM bytes per launch of the headline product kernel: rocprofv3 FETCH_SIZE 21,928.6 KiB / 0.500 (scale from a plain
+# copy of known size) + WRITE_SIZE 748.0 KiB / 1.000, from the runs summarized in profiles/gemv_m1_k5120_n17408.md
+HEADLINE_TRAFFIC_BYTES = int((21928.6 / 0.500 + 748.0) * 1024)
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA
 
 
@@ -223,8 +226,8 @@ def main():
                                "outlier-channel activations), whole op, weights rotated over >256 MB",
                    "algorithmic_bytes": b},
         "roofline": {"bound": "hbm", "achieved": round(b / kern_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(b / kern_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "rq_gemv_kernel<1>", "kernel_us": round(kern_ms * 1e3, 3)},
+                     "frac": round(b / kern_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": HEADLINE_TRAFFIC_BYTES,
+                     "kernel": "rq_gemv_kernel<1, 4>", "kernel_us": round(kern_ms * 1e3, 3)},
         "cpu_baseline": cpu,
         "parity_vs_oracle": parity,
         "extra": extra,

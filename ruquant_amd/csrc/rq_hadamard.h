@@ -125,6 +125,33 @@ __device__ __forceinline__ void fwht_pass(float *buf, int K, int lm, int ls, int
 }
 
 
+// One row of K floats (K % 4 == 0) from global memory into the padded LDS row. All of a batch's loads are issued
+// before the first LDS store: the row of a long K is several trips to memory per thread, and taken one at a time
+// each trip would cost a full memory latency.
+template <int NT>
+__device__ __forceinline__ void load_row(float *buf, const float *__restrict__ xr, int K, int tid) {
+    constexpr int kBatch = 8;
+    for (int i0 = tid * 4; i0 < K; i0 += NT * 4 * kBatch) {
+        float4 v[kBatch];
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const int i = i0 + b * NT * 4;
+            v[b] = *reinterpret_cast<const float4 *>(xr + (i < K ? i : i0));   // past the end: a harmless reload
+        }
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const int i = i0 + b * NT * 4;
+            if (i < K) {
+                float *d = buf + padi(i);      // i % 4 == 0: the four land in one run of 16
+                d[0] = v[b].x;
+                d[1] = v[b].y;
+                d[2] = v[b].z;
+                d[3] = v[b].w;
+            }
+        }
+    }
+}
+
 // all Sylvester stages of every chunk of m = 1 << lm floats of a padded row, four stages per trip through LDS
 __device__ __forceinline__ void fwht_row(float *buf, int K, int lm, int tid, int nt) {
     for (int ls = 0; ls < lm;) {

@@ -52,14 +52,7 @@ __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs 
     const int wave = tid >> 6, lane = tid & 63;
 
     const float *xr = a.x + (int64_t) t * a.ldx;
-    for (int i = tid * 4; i < K; i += kRT * 4) {
-        const float4 v = *reinterpret_cast<const float4 *>(xr + i);
-        float *d = buf + padi(i);
-        d[0] = v.x;
-        d[1] = v.y;
-        d[2] = v.z;
-        d[3] = v.w;
-    }
+    load_row<kRT>(buf, xr, K, tid);
     __syncthreads();
     fwht_row(buf, K, lm, tid, kRT);
 

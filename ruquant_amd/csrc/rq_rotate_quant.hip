@@ -50,14 +50,7 @@ __global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs
     float *g_hi = g_lo + ng;
 
     const float *xr = a.x + (int64_t) t * a.ldx;
-    for (int i = tid * 4; i < K; i += kNT * 4) {
-        const float4 v = *reinterpret_cast<const float4 *>(xr + i);
-        float *d = buf + padi(i);                // i % 4 == 0: the four land in one run of 16
-        d[0] = v.x;
-        d[1] = v.y;
-        d[2] = v.z;
-        d[3] = v.w;
-    }
+    load_row<kNT>(buf, xr, K, tid);
     __syncthreads();
 
     if (a.rotate) {
