@@ -19,12 +19,14 @@
 // accumulators every group and fold floor(k (64 Xhi + Xlo) / 16) on the vector ALU.
 //
 // Data movement: a workgroup of eight wavefronts owns 256 rows (four panels) x 128 tokens; wavefront (wr, wc) owns
-// rows 64 wr.. and tokens 64 wc.. as 4 x 4 MFMA tiles. The operands of one group (8 KiB of packed weights, 16 KiB of
+// rows 64 wr.. and tokens 64 wc.. as 4 x 4 MFMA tiles (a narrow variant for the tail of a launch: see the kernel). The operands of one group (8 KiB of packed weights, 16 KiB of
 // activation digits) go from global memory straight into LDS with global_load_lds_dwordx4 (no registers, no
 // ds_write), kStages groups deep, so a fetch has several groups of arithmetic to complete. The prepared weight
 // layout and the quantizer's output layout are exactly the LDS layouts: every wavefront-wide transfer is 1 KiB
 // contiguous on both sides.
 #include "rq_common.h"
+
+#include <stdlib.h>
 
 #pragma clang fp contract(off)
 
@@ -36,15 +38,19 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) const void global_cvoid;
 
-constexpr int kBN = 256;        // rows per workgroup (four panels)
-constexpr int kBT = 128;        // tokens per workgroup
+constexpr int kBT = 128;        // tokens per workgroup, wide tiles
+constexpr int kBTn = 32;        // tokens per workgroup, narrow tiles
 constexpr int kThreads = 512;
 constexpr int kStages = 6;      // LDS ring depth
-constexpr int kLoads = 3;       // LDS-direct loads per thread and group: 1 weight cell + 2 activation cells
+constexpr int kLoads = 3;       // LDS-direct loads per thread and step (both tile shapes)
 
+// One ring stage = 1536 cells of 16 bytes = 24 KiB.
+//   wide tile  : [0, 512)    packed weights of one group  [panel 4][half 2][row 64]
+//                [512, 1536) activation digits            [digit 2][quarter 4][token 128]
+//   narrow tile: [0, 1024)   packed weights of two groups [group 2][panel 4][half 2][row 64]
+//                [1024,1536) activation digits            [group 2][digit 2][quarter 4][token 32]
 struct Stage {
-    uint4 a[4][2][64];      // packed weights [panel][half of the group][row]: 16 bytes = 32 codes
-    uint4 b[2][4][kBT];     // activation digits [0 = lo, 1 = hi][quarter of the group][token]
+    uint4 cell[1536];
 };
 static_assert(sizeof(Stage) == 24576, "stage size");
 
@@ -58,9 +64,9 @@ __device__ __forceinline__ v4i as_v4i(const uint4 v) { return v4i{ (int) v.x, (i
 
 struct Ctx {
     const uint4 *w_src;   // this thread's weight cell of group 0
-    const uint4 *a_src;   // this thread's first activation cell of group 0
+    const uint4 *a_src;   // this thread's (first) activation cell of group 0
     size_t a_cell, a_step;
-    int wave, wr, wc, l16, quad;
+    int wave, wr, wc, l16, quad;   // wc: token half (wide) or K half (narrow)
     int ng;
 };
 
@@ -72,28 +78,48 @@ __device__ __forceinline__ void load_to_lds(const uint4 *gptr, uint4 *lds) {
     const uint32_t lds_addr = (uint32_t) (uintptr_t) (lds_void *) lds;
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                  :
-                 : "v"(gptr), "s"(lds_addr)
+                 :  "v"(gptr), "s"(lds_addr)
                  : "memory", "m0");
 }
 
-// fetch of group g into stage s: every wavefront moves three 1 KiB runs
-__device__ __forceinline__ void fetch(const Ctx &c, Stage &s, int g) {
-    const int gg = g < c.ng ? g : c.ng - 1;   // past the end: refetch the last group into a stage nobody reads
-    uint4 *a_dst = &s.a[0][0][0] + c.wave * 64;
-    uint4 *b_dst = &s.b[0][0][0] + c.wave * 64;
-    load_to_lds(c.w_src + (size_t) gg * 128, a_dst);
-    load_to_lds(c.a_src + (size_t) gg * c.a_step, b_dst);
-    load_to_lds(c.a_src + (size_t) gg * c.a_step + c.a_cell, b_dst + 512);
+// fetch of step `st` into stage s: every wavefront moves three 1 KiB runs. Groups past the end are clamped to the
+// last one (refetched into cells nobody reads).
+template <bool NARROW>
+__device__ __forceinline__ void fetch(const Ctx &c, Stage &s, int st) {
+    uint4 *dst = &s.cell[0] + c.wave * 64;
+    if (!NARROW) {
+        const int g = st < c.ng ? st : c.ng - 1;
+        load_to_lds(c.w_src + (size_t) g * 128, dst);
+        load_to_lds(c.a_src + (size_t) g * c.a_step, dst + 512);
+        load_to_lds(c.a_src + (size_t) g * c.a_step + c.a_cell, dst + 1024);
+    } else {
+        const int last = c.ng - 1;
+        const int g0 = 2 * st < last ? 2 * st : last, g1 = 2 * st + 1 < last ? 2 * st + 1 : last;
+        const int gb = 2 * st + (c.wave >> 2) < last ? 2 * st + (c.wave >> 2) : last;   // this wavefront's digit cells
+        load_to_lds(c.w_src + (size_t) g0 * 128, dst);
+        load_to_lds(c.w_src + (size_t) g1 * 128, dst + 512);
+        load_to_lds(c.a_src + (size_t) gb * c.a_step, dst + 1024);
+    }
 }
 
-template <bool HASK>
-__device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint8_t *__restrict__ k_src, int g,
-                                        v4i (&hi)[4][4], int32_t (&lo)[4][4][4]) {
+// One step of one wavefront: 64 rows x TT token tiles of 16 against one group (wide: group `st`, token half wc;
+// narrow: group 2 st + wc).
+template <bool HASK, bool NARROW>
+__device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint8_t *__restrict__ k_src, int st,
+                                        v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
+    constexpr int TT = NARROW ? 2 : 4;
+    const int g = NARROW ? 2 * st + c.wc : st;
+    if (NARROW && g >= c.ng) return;   // odd group count: the second K half sits out the last step (wave-uniform)
+    // A: quarter `quad` of the group = 8 bytes of the row's cell in half quad >> 1
+    const uint4 *a_cells = &s.cell[0] + (NARROW ? c.wc * 512 : 0) + (c.wr * 2 + (c.quad >> 1)) * 64 + c.l16;
+    // B: [digit][quarter][token]
+    const uint4 *b_cells = NARROW ? &s.cell[1024] + c.wc * 256 + c.quad * kBTn + c.l16
+                                  : &s.cell[512] + c.quad * kBT + 64 * c.wc + c.l16;
+    constexpr int kDigit = NARROW ? 4 * kBTn : 4 * kBT;   // cells between the lo and the hi plane
     v4i A[4];
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
-        // quarter `quad` of the group = 8 bytes of the row's cell in half quad >> 1
-        const uint2 pk = *(reinterpret_cast<const uint2 *>(&s.a[c.wr][c.quad >> 1][16 * rt + c.l16]) + (c.quad & 1));
+        const uint2 pk = *(reinterpret_cast<const uint2 *>(a_cells + 16 * rt) + (c.quad & 1));
         int e0, o0, e1, o1;
         widen(pk.x, e0, o0);
         widen(pk.y, e1, o1);
@@ -109,14 +135,14 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint
         }
     }
     if (!HASK) {
-        // Software pipeline over the four token tiles: the eight MFMAs of tile ct are issued back to back while the
+        // Software pipeline over the token tiles: the eight MFMAs of tile ct are issued back to back while the
         // vector ALU folds the four results of tile ct - 1, so neither unit waits for the other.
         v4i S[2][4];
 #pragma unroll
-        for (int ct = 0; ct < 5; ++ct) {
-            if (ct < 4) {
-                const v4i Blo = as_v4i(s.b[0][c.quad][64 * c.wc + 16 * ct + c.l16]);
-                const v4i Bhi = as_v4i(s.b[1][c.quad][64 * c.wc + 16 * ct + c.l16]);
+        for (int ct = 0; ct < TT + 1; ++ct) {
+            if (ct < TT) {
+                const v4i Blo = as_v4i(b_cells[16 * ct]);
+                const v4i Bhi = as_v4i(b_cells[kDigit + 16 * ct]);
 #pragma unroll
                 for (int rt = 0; rt < 4; ++rt) {
                     S[ct & 1][rt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Blo, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
@@ -130,7 +156,7 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint
                     for (int i = 0; i < 4; ++i) lo[rt][ct - 1][i] += S[(ct - 1) & 1][rt][i] >> 8;
                 }
             }
-            if (ct > 0 && ct < 4) {
+            if (ct > 0 && ct < TT) {
                 // 8 MFMAs interleaved with the 32 vector ops of the previous tile's fold: 1 MFMA, 4 VALU, ...
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
@@ -141,9 +167,9 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint
         }
     } else {
 #pragma unroll
-        for (int ct = 0; ct < 4; ++ct) {
-            const v4i Blo = as_v4i(s.b[0][c.quad][64 * c.wc + 16 * ct + c.l16]);
-            const v4i Bhi = as_v4i(s.b[1][c.quad][64 * c.wc + 16 * ct + c.l16]);
+        for (int ct = 0; ct < TT; ++ct) {
+            const v4i Blo = as_v4i(b_cells[16 * ct]);
+            const v4i Bhi = as_v4i(b_cells[kDigit + 16 * ct]);
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) {
                 const v4i H = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Bhi, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
@@ -155,43 +181,49 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint
     }
 }
 
-// One group: wait for its operands, meet the other wavefronts, refill the stage that was just released, compute.
-// At the wait, the loads this thread has issued after group g's are those of groups g+1 .. g+kStages-2.
-template <bool HASK>
+// One step: wait for its operands, meet the other wavefronts, refill the stage that was just released, compute.
+// At the wait, the loads this thread has issued after step st's are those of steps st+1 .. st+kStages-2.
+template <bool HASK, bool NARROW>
 __device__ __forceinline__ void step(const Ctx &c, const Stage &cur, Stage &refill, const uint8_t *__restrict__ k_src,
-                                     int g, v4i (&hi)[4][4], int32_t (&lo)[4][4][4]) {
+                                     int st, v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 2) * kLoads) : "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    fetch(c, refill, g + kStages - 1);
-    compute<HASK>(c, cur, k_src, g, hi, lo);
+    fetch<NARROW>(c, refill, st + kStages - 1);
+    compute<HASK, NARROW>(c, cur, k_src, st, hi, lo);
 }
 
-template <bool HASK>
+template <bool HASK, bool NARROW>
 __device__ __forceinline__ void gemm_body(const Ctx &c, Stage &s0, Stage &s1, Stage &s2, Stage &s3, Stage &s4,
-                                          Stage &s5, const uint8_t *__restrict__ k_src, v4i (&hi)[4][4],
-                                          int32_t (&lo)[4][4][4]) {
-    fetch(c, s0, 0);
-    fetch(c, s1, 1);
-    fetch(c, s2, 2);
-    fetch(c, s3, 3);
-    fetch(c, s4, 4);
-    for (int g = 0; g < c.ng; g += kStages) {
-        step<HASK>(c, s0, s5, k_src, g, hi, lo);
-        if (g + 1 < c.ng) step<HASK>(c, s1, s0, k_src, g + 1, hi, lo);
-        if (g + 2 < c.ng) step<HASK>(c, s2, s1, k_src, g + 2, hi, lo);
-        if (g + 3 < c.ng) step<HASK>(c, s3, s2, k_src, g + 3, hi, lo);
-        if (g + 4 < c.ng) step<HASK>(c, s4, s3, k_src, g + 4, hi, lo);
-        if (g + 5 < c.ng) step<HASK>(c, s5, s4, k_src, g + 5, hi, lo);
+                                          Stage &s5, const uint8_t *__restrict__ k_src,
+                                          v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
+    const int n_steps = NARROW ? (c.ng + 1) / 2 : c.ng;
+    fetch<NARROW>(c, s0, 0);
+    fetch<NARROW>(c, s1, 1);
+    fetch<NARROW>(c, s2, 2);
+    fetch<NARROW>(c, s3, 3);
+    fetch<NARROW>(c, s4, 4);
+    for (int st = 0; st < n_steps; st += kStages) {
+        step<HASK, NARROW>(c, s0, s5, k_src, st, hi, lo);
+        if (st + 1 < n_steps) step<HASK, NARROW>(c, s1, s0, k_src, st + 1, hi, lo);
+        if (st + 2 < n_steps) step<HASK, NARROW>(c, s2, s1, k_src, st + 2, hi, lo);
+        if (st + 3 < n_steps) step<HASK, NARROW>(c, s3, s2, k_src, st + 3, hi, lo);
+        if (st + 4 < n_steps) step<HASK, NARROW>(c, s4, s3, k_src, st + 4, hi, lo);
+        if (st + 5 < n_steps) step<HASK, NARROW>(c, s5, s4, k_src, st + 5, hi, lo);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the refetches of the last group before LDS is released
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the refetches of the last step before LDS is reused
 }
 
+// Wide tiles (256 rows x 128 tokens) are the efficient shape, but a launch of T of them keeps the chip busy for
+// ceil(T / 256) rounds. So the first floor(T / 256) * 256 tiles run wide, and the rest (`first_tile` onwards) run as
+// narrow tiles: the same 256 rows x 32 tokens, with the two wavefront columns taking alternate groups of K instead of
+// token halves and meeting in LDS at the end. Four times as many workgroups of a quarter of the work each.
+template <bool NARROW>
 __global__ void __launch_bounds__(kThreads)
 rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                const int32_t *__restrict__ flags, const uint4 *__restrict__ act8, const float *__restrict__ u,
-               float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng, int n_panels, int n_row_tiles,
-               int n_tok_tiles) {
+               float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng, int n_panels, int n_tok_tiles,
+               int first_tile, int n_tiles) {
     // one array per stage: the compiler tracks LDS-direct loads per destination object
     __shared__ Stage s0;
     __shared__ Stage s1;
@@ -199,15 +231,26 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     __shared__ Stage s3;
     __shared__ Stage s4;
     __shared__ Stage s5;
+    constexpr int TT = NARROW ? 2 : 4;
 
-    // Workgroups go to the eight XCDs round robin. Give every XCD a contiguous run of row tiles with the token
+    // Workgroups go to the eight XCDs round robin. Wide: give every XCD a contiguous run of row tiles with the token
     // tiles running fastest, so the workgroups resident on one XCD share weight and activation tiles in its L2.
-    const int total = n_row_tiles * n_tok_tiles;
-    int v = blockIdx.x;
-    const int per_xcd = total / 8;
-    if (v < per_xcd * 8) v = (v & 7) * per_xcd + (v >> 3);
+    // Narrow: the four token quarters of a tile sit 8 apart in dispatch order (same XCD, close in time).
+    int v, t0;
+    if (!NARROW) {
+        v = blockIdx.x;
+        const int per_xcd = n_tiles / 8;
+        if (v < per_xcd * 8) v = (v & 7) * per_xcd + (v >> 3);
+        t0 = 0;
+    } else {
+        const int b = blockIdx.x;
+        v = first_tile + (b >> 5) * 8 + (b & 7);
+        t0 = ((b >> 3) & 3) * kBTn;
+        if (v >= n_tiles) return;
+    }
     const int row_tile = v / n_tok_tiles, tok_tile = v - row_tile * n_tok_tiles;
-    const int panel0 = row_tile * 4, t0 = tok_tile * kBT;
+    const int panel0 = row_tile * 4;
+    t0 += tok_tile * kBT;
 
     const int tid = threadIdx.x;
     Ctx c;
@@ -217,23 +260,29 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     c.l16 = tid & 15;
     c.quad = (tid & 63) >> 4;
     c.ng = ng;
-    // weights: thread tid moves cell tid of the tile's 512 (panel = tid >> 7, half = (tid >> 6) & 1, row = tid & 63);
+    // weights: thread tid moves cell tid of a group's 512 (panel = tid >> 7, half = (tid >> 6) & 1, row = tid & 63);
     // panels past the tensor read panel n_panels - 1 again (their outputs are never stored)
     const int w_panel = min(panel0 + (tid >> 7), n_panels - 1);
     c.w_src = codes + (size_t) w_panel * ng * 128 + (tid & 127);
-    // activations: the tile of one group is 1024 cells [digit][quarter][token]; thread tid moves cells tid and
-    // tid + 512 (digit = cell >> 9, quarter = (cell >> 7) & 3, token = cell & 127)
-    c.a_src = act8 + (size_t) (tid >> 7) * Mp + t0 + (tid & 127);
-    c.a_cell = (size_t) 4 * Mp;   // + 512 cells = the other digit
     c.a_step = (size_t) 8 * Mp;   // cells per group
+    c.a_cell = (size_t) 4 * Mp;   // the other digit
+    if (!NARROW) {
+        // the tile of one group is 1024 cells [digit][quarter][token]; thread tid moves cells tid and tid + 512
+        // (digit = cell >> 9, quarter = (cell >> 7) & 3, token = cell & 127)
+        c.a_src = act8 + (size_t) (tid >> 7) * Mp + t0 + (tid & 127);
+    } else {
+        // two groups of 256 cells [digit][quarter][token 32]; thread tid moves cell tid & 255 of group tid >> 8
+        // (the group is added per step: it is uniform per wavefront)
+        c.a_src = act8 + (size_t) ((tid >> 5) & 7) * Mp + t0 + (tid & 31);
+    }
     const uint8_t *k_src = kmul + (size_t) min(panel0 + c.wr, n_panels - 1) * ng * kPanelRows + 4 * c.quad;
 
-    v4i hi[4][4];
-    int32_t lo[4][4][4];
+    v4i hi[4][TT];
+    int32_t lo[4][TT][4];
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
 #pragma unroll
-        for (int ct = 0; ct < 4; ++ct) {
+        for (int ct = 0; ct < TT; ++ct) {
             hi[rt][ct] = v4i{ 0, 0, 0, 0 };
 #pragma unroll
             for (int i = 0; i < 4; ++i) lo[rt][ct][i] = 0;
@@ -241,36 +290,70 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     }
 
     if (flags[0] & 1) {
-        gemm_body<true>(c, s0, s1, s2, s3, s4, s5, k_src, hi, lo);
+        gemm_body<true, NARROW>(c, s0, s1, s2, s3, s4, s5, k_src, hi, lo);
     } else {
-        gemm_body<false>(c, s0, s1, s2, s3, s4, s5, k_src, hi, lo);
+        gemm_body<false, NARROW>(c, s0, s1, s2, s3, s4, s5, k_src, hi, lo);
+    }
+
+    int32_t tot[4][TT][4];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+#pragma unroll
+        for (int ct = 0; ct < TT; ++ct) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) tot[rt][ct][i] = (hi[rt][ct][i] >> 2) + lo[rt][ct][i];
+        }
+    }
+    if (NARROW) {
+        // the odd-group half hands its totals to the even-group half through LDS (the stages are free now):
+        // 32 values per lane, 16 KiB per pair of row tiles
+        __syncthreads();
+        int32_t *xch0 = reinterpret_cast<int32_t *>(&s0.cell[0]) + (c.wr * 64 + (tid & 63));
+        int32_t *xch1 = reinterpret_cast<int32_t *>(&s1.cell[0]) + (c.wr * 64 + (tid & 63));
+        if (c.wc == 1) {
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+#pragma unroll
+                for (int ct = 0; ct < TT; ++ct) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) (rt < 2 ? xch0 : xch1)[(((rt & 1) * TT + ct) * 4 + i) * 256] = tot[rt][ct][i];
+                }
+            }
+        }
+        __syncthreads();
+        if (c.wc == 1) return;
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+#pragma unroll
+            for (int ct = 0; ct < TT; ++ct) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) tot[rt][ct][i] += (rt < 2 ? xch0 : xch1)[(((rt & 1) * TT + ct) * 4 + i) * 256];
+            }
+        }
     }
 
     // epilogue (reference patch line 176): y = ((float(total) * 16) * u) * s_w, total = 4 Xhi + sum of floors
 #pragma unroll
-    for (int ct = 0; ct < 4; ++ct) {
-        const int t = t0 + 64 * c.wc + 16 * ct + c.l16;
+    for (int ct = 0; ct < TT; ++ct) {
+        const int t = t0 + (NARROW ? 0 : 64 * c.wc) + 16 * ct + c.l16;
         if (t >= M) continue;
         const float ut = u[t];
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) {
             const int64_t n = (int64_t) (panel0 + c.wr) * kPanelRows + 16 * rt + 4 * c.quad;
             float *dst = y + (int64_t) t * ldy + n;
-            int32_t tot[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) tot[i] = (hi[rt][ct][i] >> 2) + lo[rt][ct][i];
             if (n + 3 < N && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
                 const float4 sw = *reinterpret_cast<const float4 *>(s_w + n);
                 float4 o;
-                o.x = (((float) tot[0] * 16.0f) * ut) * sw.x;
-                o.y = (((float) tot[1] * 16.0f) * ut) * sw.y;
-                o.z = (((float) tot[2] * 16.0f) * ut) * sw.z;
-                o.w = (((float) tot[3] * 16.0f) * ut) * sw.w;
+                o.x = (((float) tot[rt][ct][0] * 16.0f) * ut) * sw.x;
+                o.y = (((float) tot[rt][ct][1] * 16.0f) * ut) * sw.y;
+                o.z = (((float) tot[rt][ct][2] * 16.0f) * ut) * sw.z;
+                o.w = (((float) tot[rt][ct][3] * 16.0f) * ut) * sw.w;
                 *reinterpret_cast<float4 *>(dst) = o;
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    if (n + i < N) dst[i] = (((float) tot[i] * 16.0f) * ut) * s_w[n + i];
+                    if (n + i < N) dst[i] = (((float) tot[rt][ct][i] * 16.0f) * ut) * s_w[n + i];
                 }
             }
         }
@@ -283,12 +366,27 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     const uint8_t *p = a.prepared;
     const int n_row_tiles = (a.L.n_panels + 3) / 4;
     const int n_tok_tiles = a.Mp / kBT;
-    hipLaunchKernelGGL(rq_gemm_kernel, dim3(n_row_tiles * n_tok_tiles), dim3(kThreads), 0, stream,
-                       reinterpret_cast<const uint4 *>(p + a.L.off_codes),
-                       reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,
-                       reinterpret_cast<const int32_t *>(p + a.L.off_flags),
-                       reinterpret_cast<const uint4 *>(a.act8), a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng,
-                       a.L.n_panels, n_row_tiles, n_tok_tiles);
+    const int n_tiles = n_row_tiles * n_tok_tiles;
+    static const int force = getenv("RQ_GEMM_NARROW") ? atoi(getenv("RQ_GEMM_NARROW")) : -1;   // 0: never, 1: always
+    const int kCUs = 256;
+    int n_wide = n_tiles / kCUs * kCUs;          // whole rounds of the chip
+    if (force == 0) n_wide = n_tiles;
+    if (force == 1) n_wide = 0;
+    const uint4 *codes = reinterpret_cast<const uint4 *>(p + a.L.off_codes);
+    const float *s_w = reinterpret_cast<const float *>(p + a.L.off_sw);
+    const int32_t *flags = reinterpret_cast<const int32_t *>(p + a.L.off_flags);
+    const uint4 *act8 = reinterpret_cast<const uint4 *>(a.act8);
+    if (n_wide > 0) {
+        hipLaunchKernelGGL(rq_gemm_kernel<false>, dim3(n_wide), dim3(kThreads), 0, stream, codes, s_w,
+                           p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
+                           n_tok_tiles, 0, n_wide);
+    }
+    if (n_wide < n_tiles) {
+        const int rest = n_tiles - n_wide;
+        hipLaunchKernelGGL(rq_gemm_kernel<true>, dim3((rest + 7) / 8 * 32), dim3(kThreads), 0, stream, codes, s_w,
+                           p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
+                           n_tok_tiles, n_wide, n_tiles);
+    }
     return hipGetLastError();
 }
 
