@@ -181,16 +181,89 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint
     }
 }
 
-// One step: wait for its operands, meet the other wavefronts, refill the stage that was just released, compute.
-// At the wait, the loads this thread has issued after step st's are those of steps st+1 .. st+kStages-2.
+// Two groups of a wide tile at once (the fast path: no weight multipliers). With both groups' low-digit sums at
+// hand the fold is lo += (Sa >> 8) + (Sb >> 8): two shifts and ONE three-operand add, a quarter fewer vector
+// instructions than group by group. Software pipeline in units of one 16 x 16 tile (x two groups = 4 MFMAs): the
+// MFMAs of unit i are issued while the vector ALU folds unit i - 1.
+template <bool NARROW>
+__device__ __forceinline__ void compute_pair(const Ctx &c, const Stage &sa, const Stage &sb, bool both,
+                                             v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
+    constexpr int TT = NARROW ? 2 : 4;
+    constexpr int kDigit = NARROW ? 4 * kBTn : 4 * kBT;   // cells between the lo and the hi plane
+    const int a_off = (NARROW ? c.wc * 512 : 0) + (c.wr * 2 + (c.quad >> 1)) * 64 + c.l16;
+    const int b_off = NARROW ? 1024 + c.wc * 256 + c.quad * kBTn + c.l16 : 512 + c.quad * kBT + 64 * c.wc + c.l16;
+    v4i Aa[4], Ab[4];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+        const uint2 pa = *(reinterpret_cast<const uint2 *>(&sa.cell[a_off + 16 * rt]) + (c.quad & 1));
+        const uint2 pb = *(reinterpret_cast<const uint2 *>(&sb.cell[a_off + 16 * rt]) + (c.quad & 1));
+        int e0, o0, e1, o1;
+        widen(pa.x, e0, o0);
+        widen(pa.y, e1, o1);
+        Aa[rt] = v4i{ e0, o0, e1, o1 };
+        widen(pb.x, e0, o0);
+        widen(pb.y, e1, o1);
+        Ab[rt] = v4i{ e0, o0, e1, o1 };
+    }
+    if (!both) {   // odd group count: the last pair has one group; zero weights make the second one vanish
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) Ab[rt] = v4i{ 0, 0, 0, 0 };
+    }
+    v4i Sa[2], Sb[2];
+    v4i B[2][4];   // [buffer][lo a, hi a, lo b, hi b] of one token tile; the next tile's are fetched a unit ahead
+    auto load_b = [&](int buf, int ct) {
+        B[buf][0] = as_v4i(sa.cell[b_off + 16 * ct]);
+        B[buf][1] = as_v4i(sa.cell[b_off + kDigit + 16 * ct]);
+        B[buf][2] = as_v4i(sb.cell[b_off + 16 * ct]);
+        B[buf][3] = as_v4i(sb.cell[b_off + kDigit + 16 * ct]);
+    };
+    load_b(0, 0);
+#pragma unroll
+    for (int un = 0; un < 4 * TT + 1; ++un) {
+        const int ct = un >> 2, rt = un & 3;
+        if (rt == 0) __builtin_amdgcn_sched_barrier(0);   // keeps the LDS reads of later tiles from piling up early
+        if (un < 4 * TT) {
+            if (rt == 0 && ct < TT - 1) load_b((ct + 1) & 1, ct + 1);
+            Sa[un & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aa[rt], B[ct & 1][0], v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+            Sb[un & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ab[rt], B[ct & 1][2], v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+            hi[rt][ct] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aa[rt], B[ct & 1][1], hi[rt][ct], 0, 0, 0);
+            hi[rt][ct] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ab[rt], B[ct & 1][3], hi[rt][ct], 0, 0, 0);
+        }
+        if (un > 0) {
+            const int pct = (un - 1) >> 2, prt = (un - 1) & 3;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) lo[prt][pct][i] += (Sa[(un - 1) & 1][i] >> 8) + (Sb[(un - 1) & 1][i] >> 8);
+        }
+        if (un > 0 && un < 4 * TT) {
+            // 4 MFMAs interleaved with the 12 vector ops of the previous unit's fold
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // VALU
+            }
+        }
+    }
+}
+
+// One pair of steps: wait for their operands, meet the other wavefronts, refill the two stages that were just
+// released, compute. At the wait, the loads this thread has issued after this pair's are those of the next pair.
 template <bool HASK, bool NARROW>
-__device__ __forceinline__ void step(const Ctx &c, const Stage &cur, Stage &refill, const uint8_t *__restrict__ k_src,
-                                     int st, v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 2) * kLoads) : "memory");
+__device__ __forceinline__ void pair_step(const Ctx &c, const Stage &cur0, const Stage &cur1, Stage &refill0,
+                                          Stage &refill1, const uint8_t *__restrict__ k_src, int st, int n_steps,
+                                          v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoads) : "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    fetch<NARROW>(c, refill, st + kStages - 1);
-    compute<HASK, NARROW>(c, cur, k_src, st, hi, lo);
+    fetch<NARROW>(c, refill0, st + 4);
+    fetch<NARROW>(c, refill1, st + 5);
+    if constexpr (!HASK) {
+        // narrow tiles: the wavefront's second group exists if 2 (st + 1) + wc < ng
+        const bool both = NARROW ? 2 * (st + 1) + c.wc < c.ng : st + 1 < n_steps;
+        if (!NARROW || 2 * st + c.wc < c.ng) compute_pair<NARROW>(c, cur0, cur1, both, hi, lo);
+    } else {
+        compute<HASK, NARROW>(c, cur0, k_src, st, hi, lo);
+        if (st + 1 < n_steps) compute<HASK, NARROW>(c, cur1, k_src, st + 1, hi, lo);
+    }
 }
 
 template <bool HASK, bool NARROW>
@@ -202,16 +275,12 @@ __device__ __forceinline__ void gemm_body(const Ctx &c, Stage &s0, Stage &s1, St
     fetch<NARROW>(c, s1, 1);
     fetch<NARROW>(c, s2, 2);
     fetch<NARROW>(c, s3, 3);
-    fetch<NARROW>(c, s4, 4);
     for (int st = 0; st < n_steps; st += kStages) {
-        step<HASK, NARROW>(c, s0, s5, k_src, st, hi, lo);
-        if (st + 1 < n_steps) step<HASK, NARROW>(c, s1, s0, k_src, st + 1, hi, lo);
-        if (st + 2 < n_steps) step<HASK, NARROW>(c, s2, s1, k_src, st + 2, hi, lo);
-        if (st + 3 < n_steps) step<HASK, NARROW>(c, s3, s2, k_src, st + 3, hi, lo);
-        if (st + 4 < n_steps) step<HASK, NARROW>(c, s4, s3, k_src, st + 4, hi, lo);
-        if (st + 5 < n_steps) step<HASK, NARROW>(c, s5, s4, k_src, st + 5, hi, lo);
+        pair_step<HASK, NARROW>(c, s0, s1, s4, s5, k_src, st, n_steps, hi, lo);
+        if (st + 2 < n_steps) pair_step<HASK, NARROW>(c, s2, s3, s0, s1, k_src, st + 2, n_steps, hi, lo);
+        if (st + 4 < n_steps) pair_step<HASK, NARROW>(c, s4, s5, s2, s3, k_src, st + 4, n_steps, hi, lo);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the refetches of the last step before LDS is reused
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the refetches of the last steps before LDS is reused
 }
 
 // Wide tiles (256 rows x 128 tokens) are the efficient shape, but a launch of T of them keeps the chip busy for
