@@ -126,16 +126,19 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     q.m = m;
     q.scale = 1.0f / sqrtf((float) q.n_rot);
     q.clip = clip;
-    q.mode = gemm ? kActI8 : kActStats;
+    // Skinny batches with a long Paley stage: one workgroup per token would leave most of the chip idle for tens of
+    // microseconds, so the rotation runs spread over workgroups (ranges out) and a second small kernel quantizes.
+    const bool two_step = path == kPathSkinny && q.rotate && p >= 44 && (m & 63) == 0;
+    q.mode = gemm && !two_step ? kActI8 : kActStats;
     q.u = reinterpret_cast<float *>(wsb + W.off_u);
-    q.act = reinterpret_cast<uint32_t *>(wsb + W.off_act);
+    q.act = reinterpret_cast<uint32_t *>(wsb + W.off_i8);
     // token stride of the digit planes: the GEMM pads to its tile; the skinny kernel wants them dense (a padded
     // plane would put all of its reads on the few L2 channels that the used 256 bytes of every 2 KB map to)
     const int act_mp = path == kPathSkinny ? (int) ((M + 15) / 16 * 16) : (int) W.Mp;
     q.Mp = act_mp;
     const float *gemv_x = x;      // what the GEMV quantizes from: the rotated rows, or x itself for W4A4
     int64_t gemv_ldx = ldx;
-    if (!gemm) {
+    if (!gemm || two_step) {
         q.lohi = reinterpret_cast<float *>(wsb + W.off_lohi);
         q.rpart = reinterpret_cast<float *>(wsb + W.off_rpart);
         if (q.rotate) {
@@ -144,6 +147,8 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             gemv_x = q.out_f32;
             gemv_ldx = K;
         }
+    }
+    if (!gemm) {
         q.zero_ptr = reinterpret_cast<int32_t *>(wsb + W.off_tot);
         // only the token slots this call can touch: [min(M, 8)][padded rows] cells of two ints
         const int64_t slots = M < kGemvTokens ? M : kGemvTokens;
@@ -154,8 +159,12 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     }
     hipError_t e = hipSuccess;
     if (stages & 1) {
-        e = gemm ? launch_rotate_quant(q, stream) : launch_rotate_stats(q, stream);
+        e = q.mode == kActI8 ? launch_rotate_quant(q, stream) : launch_rotate_stats(q, stream);
         if (e != hipSuccess) return (int) e;
+        if (two_step) {
+            e = launch_quantize_digits(q, stream);
+            if (e != hipSuccess) return (int) e;
+        }
     }
     if (!(stages & 2)) return 0;
 
@@ -165,7 +174,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             SkinnyArgs g;
             g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
             g.L = L;
-            g.act8 = wsb + W.off_act;
+            g.act8 = wsb + W.off_i8;
             g.u = q.u;
             g.y = y[i];
             g.ldy = ldy[i];
@@ -178,7 +187,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             GemmArgs g;
             g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
             g.L = L;
-            g.act8 = wsb + W.off_act;
+            g.act8 = wsb + W.off_i8;
             g.u = q.u;
             g.y = y[i];
             g.ldy = ldy[i];

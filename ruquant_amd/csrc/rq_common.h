@@ -65,15 +65,16 @@ inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
 //   act    : GEMV path (M <= 32): the rotated activations as fp32 rows [M][K] followed by the clipped group
 //            ranges [M][ng][2] (lo, hi) and [M][32] partial maxima of hi - lo; every GEMV workgroup quantizes
 //            the K slice it consumes itself.
-//            GEMM path: two int8 digit planes of m (q - z), [g][digit][quarter][Mp][16 bytes], in the byte order
-//            the weight unpack produces.
+//            MFMA paths: two int8 digit planes of m (q - z), [g][digit][quarter][Mp][16 bytes], in the byte order
+//            the weight unpack produces (for M <= 64 they follow the fp32 form, which the skinny path may use as
+//            an intermediate).
 //   cells  : split-K cells [8 or 64 tokens][n_panels * 64], 64 bits each: arrival count above bit 48, exact sum
 //            below.
 // ---------------------------------------------------------------------------------------------------
 struct WorkspaceLayout {
     int64_t Mp;       // tokens padded to the GEMM tile
     int     chunks;   // ceil(M / 8)
-    size_t  off_u, off_act, off_lohi, off_rpart, off_tot, bytes;
+    size_t  off_u, off_act, off_lohi, off_rpart, off_i8, off_tot, bytes;
     size_t  tot_ints;
 };
 
@@ -95,7 +96,9 @@ inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
     const size_t rpart = (size_t) M * kRangeParts * sizeof(float);
     W.off_rpart = W.off_lohi + align_up(lohi, 256);
     const size_t gemv_form = align_up(rows, 256) + align_up(lohi, 256) + align_up(rpart, 256);
-    off = align_up(off + (small && gemv_form > act_i8 ? gemv_form : act_i8), 256);
+    // small batches may use both forms in one call (rotation with ranges first, digit planes from those)
+    W.off_i8 = small ? off + gemv_form : off;
+    off = align_up(off + (small ? gemv_form + act_i8 : act_i8), 256);
     W.tot_ints = (size_t) 2 * (M <= kGemvTokens ? kGemvTokens : kSkinnyTokens) * n_panels * kPanelRows;
     W.off_tot = off;
     off = align_up(off + W.tot_ints * sizeof(int32_t), 256);
@@ -140,6 +143,8 @@ hipError_t launch_rotate_quant(const RotQuantArgs &a, hipStream_t stream);
 // Activation side of the GEMV path: like launch_rotate_quant with mode kActStats, but spreads one token over
 // several workgroups when the rotation allows it (decode latency).
 hipError_t launch_rotate_stats(const RotQuantArgs &a, hipStream_t stream);
+// digit planes (kActI8 form) from the outputs of launch_rotate_stats: rows in out_f32, ranges in lohi / rpart
+hipError_t launch_quantize_digits(const RotQuantArgs &a, hipStream_t stream);
 
 struct GemvArgs {
     const uint8_t  *prepared;

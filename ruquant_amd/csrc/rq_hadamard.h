@@ -132,11 +132,11 @@ template <int NT>
 __device__ __forceinline__ void load_row(float *buf, const float *__restrict__ xr, int K, int tid) {
     constexpr int kBatch = 8;
     for (int i0 = tid * 4; i0 < K; i0 += NT * 4 * kBatch) {
-        float4 v[kBatch];
+        float4 v[kBatch] = {};
 #pragma unroll
         for (int b = 0; b < kBatch; ++b) {
             const int i = i0 + b * NT * 4;
-            v[b] = *reinterpret_cast<const float4 *>(xr + (i < K ? i : i0));   // past the end: a harmless reload
+            if (i < K) v[b] = *reinterpret_cast<const float4 *>(xr + i);
         }
 #pragma unroll
         for (int b = 0; b < kBatch; ++b) {

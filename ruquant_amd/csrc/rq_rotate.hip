@@ -31,8 +31,9 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 template <int P>
-__global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs a, int slabs) {
+__global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs a, int slabs, int parts) {
     extern __shared__ __align__(16) float buf[];
+    __shared__ float s_rmax[kRT / 64];
 
     const int tid = threadIdx.x;
     if ((int) blockIdx.x >= a.token_blocks) {
@@ -46,7 +47,11 @@ __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs 
         return;
     }
 
-    const int t = blockIdx.x / slabs, slab = blockIdx.x - t * slabs;
+    // workgroup = (token, slab of 64 columns, part): the slab's Paley items are dealt round-robin to `parts`
+    // workgroups, so that a wavefront has one or two of them
+    const int per_token = slabs * parts;
+    const int t = blockIdx.x / per_token, sp = blockIdx.x - t * per_token;
+    const int slab = sp / parts, part = sp - slab * parts;
     const int K = a.K, m = a.m, ng = K / kGroup;
     const int lm = __ffs(m) - 1;
     const int wave = tid >> 6, lane = tid & 63;
@@ -63,7 +68,7 @@ __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs 
     if constexpr (P == 1) {
         // no Paley stage: the slab is a share of the row's runs of 64
         const int runs = K >> 6;
-        for (int r = slab * (kRT / 64) + wave; r < runs; r += slabs * (kRT / 64)) {
+        for (int r = sp * (kRT / 64) + wave; r < runs; r += per_token * (kRT / 64)) {
             const int idx = 64 * r + lane;
             const float v = buf[padi(idx)] * a.scale;
             out[idx] = v;
@@ -75,15 +80,11 @@ __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs 
             rmax = fmaxf(rmax, hi - lo);
         }
     } else {
-        // wave-items = (rotation block, slice of four output chunks) for this slab's 64 columns; a wavefront takes a
-        // contiguous block of items so that it stays in one slice's straight-line code where it can
+        // wave-items = (rotation block, slice of four output chunks) for this slab's 64 columns
         const int n_rb = K / a.n_rot;
         const int n_items = n_rb * (P / 4);
-        const int per_wave = (n_items + kRT / 64 - 1) / (kRT / 64);
         const int pm = m + (m >> 4);
-        for (int it = 0; it < per_wave; ++it) {
-            const int wi = wave * per_wave + it;
-            if (wi >= n_items) break;
+        for (int wi = part + parts * wave; wi < n_items; wi += parts * (kRT / 64)) {
             const int s = wi / n_rb, rb = wi - s * n_rb;
             const int b0 = rb * a.n_rot + 64 * slab + lane;
             const float *src = buf + padi(b0);
@@ -106,9 +107,64 @@ __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs 
             }
         }
     }
-    // slot (slab, wave) of the token's partial maxima; slots nobody owns are written as zero by slab 0
-    if (lane == 0) a.rpart[(size_t) t * kRangeParts + slab * (kRT / 64) + wave] = rmax;
-    if (slab == 0 && tid >= slabs * (kRT / 64) && tid < kRangeParts) a.rpart[(size_t) t * kRangeParts + tid] = 0.0f;
+    // one slot of the token's partial maxima per workgroup; slots nobody owns are written as zero by the first one
+    if (lane == 0) s_rmax[wave] = rmax;
+    __syncthreads();
+    if (tid == 0) {
+        float r = s_rmax[0];
+#pragma unroll
+        for (int i = 1; i < kRT / 64; ++i) r = fmaxf(r, s_rmax[i]);
+        a.rpart[(size_t) t * kRangeParts + sp] = r;
+    }
+    if (sp == 0 && tid >= per_token && tid < kRangeParts) a.rpart[(size_t) t * kRangeParts + tid] = 0.0f;
+}
+
+// The activation quantizer for tokens whose rotated rows and group ranges already exist (written by the kernel
+// above): token unit from the partial range maxima, then per group the multiplier and zero point and per value the
+// code, emitted as the two int8 digits of m (q - z) in the layout of the MFMA kernels. A thread per code word; same
+// fp32 operations in the same order as the one-workgroup quantizer (reference patch lines 2639-2679).
+__global__ void __launch_bounds__(kRT) rq_quantize_digits_kernel(const RotQuantArgs a, int blocks_per_token) {
+    const int tid = threadIdx.x;
+    const int t = blockIdx.x / blocks_per_token;
+    const int w = (blockIdx.x - t * blocks_per_token) * kRT + tid;
+    const int lane = tid & 63;
+    float R = wave_max(lane < kRangeParts ? a.rpart[(size_t) t * kRangeParts + lane] : 0.0f);
+    if (R == 0.0f) R = 2.0f;
+    const float u = R / 3825.0f;  // 15 * 255
+    if (w == 0) a.u[t] = u;
+    if (w >= (a.K >> 3)) return;
+    const int g = w >> 3;
+    const float2 lh = reinterpret_cast<const float2 *>(a.lohi)[(size_t) t * (a.K / kGroup) + g];
+    const int mg = (int) fminf(fmaxf(ceilf(((lh.y - lh.x) * 255.0f) / R), 1.0f), 255.0f);
+    const float inv = 1.0f / ((float) mg * u);
+    const float zf = fminf(fmaxf(rintf(-lh.x * inv), 0.0f), 15.0f);
+    const int z = (int) zf;
+    const float4 *src = reinterpret_cast<const float4 *>(a.out_f32 + (int64_t) t * a.ldo + 8 * w);
+    const float4 v0 = src[0], v1 = src[1];
+    const float f[8] = { v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w };
+    uint32_t lo_e = 0, lo_o = 0, hi_e = 0, hi_o = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int q = (int) fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
+        // p = m (q - z), |p| <= 3825, as two balanced int8 digits p = 64 hi + lo, lo in [-32, 31]; bytes in the
+        // order the weight unpack yields: the even codes of the word, then the odd codes
+        const int p = mg * (q - z);
+        const int lo = ((p + 32) & 63) - 32;
+        const int hi = (p - lo) >> 6;
+        const int sh = 8 * (j >> 1);
+        if (j & 1) {
+            lo_o |= (uint32_t) (lo & 0xFF) << sh;
+            hi_o |= (uint32_t) (hi & 0xFF) << sh;
+        } else {
+            lo_e |= (uint32_t) (lo & 0xFF) << sh;
+            hi_e |= (uint32_t) (hi & 0xFF) << sh;
+        }
+    }
+    // [group][digit][quarter of the group][token][16 bytes]
+    const size_t cell = (((size_t) g * 2 + 0) * 4 + ((w & 7) >> 1)) * a.Mp + t;
+    uint32_t *dst = a.act + cell * 4 + (w & 1) * 2;
+    *reinterpret_cast<uint2 *>(dst) = make_uint2(lo_e, lo_o);
+    *reinterpret_cast<uint2 *>(dst + (size_t) 16 * a.Mp) = make_uint2(hi_e, hi_o);
 }
 
 template <int P>
@@ -122,12 +178,16 @@ hipError_t launch_slab(const RotQuantArgs &a, hipStream_t stream) {
     }
     // one slab per 64 columns of a chunk; without a Paley stage, a few workgroups share the row's runs
     int slabs = P > 1 ? a.m / 64 : (a.K >= 4096 ? 4 : 1);
-    if (slabs * (kRT / 64) > kRangeParts) return launch_rotate_quant(a, stream);   // more slabs than range slots
+    // enough parts that a wavefront gets one Paley item, within the token's range slots
+    const int n_items = P > 1 ? (a.K / a.n_rot) * (P / 4) : 0;
+    int parts = P > 1 ? (n_items + kRT / 64 - 1) / (kRT / 64) : 1;
+    if (slabs > kRangeParts) return launch_rotate_quant(a, stream);   // more slabs than range slots
+    while (parts > 1 && slabs * parts > kRangeParts) --parts;
     const int zero_blocks = (int) ((a.zero_ints + (int64_t) kRT * 4 - 1) / ((int64_t) kRT * 4));
     RotQuantArgs b = a;
-    b.token_blocks = a.M * slabs;
+    b.token_blocks = a.M * slabs * parts;
     const size_t lds = (size_t) (a.K + (a.K >> 4) + 1) * sizeof(float);
-    hipLaunchKernelGGL((rq_rotate_slab_kernel<P>), dim3(b.token_blocks + zero_blocks), dim3(kRT), lds, stream, b, slabs);
+    hipLaunchKernelGGL((rq_rotate_slab_kernel<P>), dim3(b.token_blocks + zero_blocks), dim3(kRT), lds, stream, b, slabs, parts);
     return hipGetLastError();
 }
 
@@ -136,7 +196,7 @@ hipError_t launch_slab(const RotQuantArgs &a, hipStream_t stream) {
 hipError_t launch_rotate_stats(const RotQuantArgs &a, hipStream_t stream) {
     // The slab kernel needs whole groups per (chunk, slab): chunks that are a multiple of 64 long. Everything else,
     // and unrotated activations (ranges only), goes through the one-workgroup-per-token kernel.
-    if (!a.rotate || (a.m & 63) != 0 || a.M > 16) return launch_rotate_quant(a, stream);
+    if (!a.rotate || (a.m & 63) != 0 || a.M > kSkinnyTokens) return launch_rotate_quant(a, stream);
     switch (a.p) {
         case 1:  return launch_slab<1>(a, stream);
         case 12: return launch_slab<12>(a, stream);
@@ -144,6 +204,12 @@ hipError_t launch_rotate_stats(const RotQuantArgs &a, hipStream_t stream) {
         case 68: return launch_slab<68>(a, stream);
         default: return launch_rotate_quant(a, stream);
     }
+}
+
+hipError_t launch_quantize_digits(const RotQuantArgs &a, hipStream_t stream) {
+    const int bpt = ((a.K >> 3) + kRT - 1) / kRT;
+    hipLaunchKernelGGL(rq_quantize_digits_kernel, dim3(a.M * bpt), dim3(kRT), 0, stream, a, bpt);
+    return hipGetLastError();
 }
 
 }  // namespace rq

@@ -24,7 +24,10 @@ constexpr int kNT = 512;  // threads per token workgroup
 using namespace had;
 
 template <int P, bool SLICED>
-__global__ void __launch_bounds__(kNT) rq_rotate_quant_kernel(const RotQuantArgs a) {
+// Registers are capped so that two workgroups (p >= 44: long columns, long rows) or three fit a compute unit: the
+// stages of one token are separated by barriers, and it is the other workgroups that keep the vector ALU busy. (The
+// sliced variant serves small batches, where occupancy is not the limit.)
+__global__ void __launch_bounds__(kNT, SLICED ? 2 : (P >= 44 ? 4 : 6)) rq_rotate_quant_kernel(const RotQuantArgs a) {
     extern __shared__ __align__(16) float smem[];
     __shared__ float s_red[kNT / 64];
 
