@@ -15,7 +15,7 @@
 // The per-group fold, the exact int32 total and the fp32 epilogue are those of ggml_vec_dot_w4a4_a4 (lines 148-177):
 //     total += (k * m_g * (acc_g + (8 - z_g) * colsum_g)) >> 4;   y = ((float(total) * 16) * u) * s_w.
 // colsum_g is recomputed from the codes (dot8 against 0x11111111) instead of being stored.
-#include "rq_common.h"
+#include "rq_hadamard.h"
 
 #include <stdlib.h>
 
@@ -152,7 +152,7 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
             }
         }
     }
-    __syncthreads();
+    had::lds_barrier();   // not __syncthreads(): the weight loads stay in flight across the prologue
 
     // ---- per (group of the slice, token): multiplier, 1 / (m u), zero point (reference lines 2662-2665)
     for (int gt = tid; gt < n_gt; gt += NT) {
@@ -166,7 +166,7 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
         s_zf[gt] = zf;
         s_mz[gt] = mg | ((8 - (int) zf) & 0xFF) << 8;
     }
-    __syncthreads();
+    had::lds_barrier();
 
     // ---- codes: a thread per code word (8 values), q = clamp(rint(x * inv) + z, 0, 15) (lines 2670-2675)
     for (int id = tid; id < n_words; id += NT) {
@@ -188,7 +188,7 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
         }
         s_act[id] = word;
     }
-    __syncthreads();
+    had::lds_barrier();
 
     // ---- the product
     const bool hask = *reinterpret_cast<const volatile int32_t *>(flags) & 1;

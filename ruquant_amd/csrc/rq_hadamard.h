@@ -125,6 +125,15 @@ __device__ __forceinline__ void fwht_pass(float *buf, int K, int lm, int ls, int
 }
 
 
+// Workgroup barrier for data that travels through LDS only: waits for this wavefront's LDS operations, not for its
+// outstanding global loads (which __syncthreads() would also drain, stalling a kernel that keeps weight loads in
+// flight across its prologue).
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // One row of K floats (K % 4 == 0) from global memory into the padded LDS row. All of a batch's loads are issued
 // before the first LDS store: the row of a long K is several trips to memory per thread, and taken one at a time
 // each trip would cost a full memory latency.
