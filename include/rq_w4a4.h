@@ -132,6 +132,28 @@ int rq_w4a4_hadamard(const float *x_dev, int64_t ldx, int64_t M, int64_t K, int6
 int rq_w4a4_quantize_act(int type, const float *x_dev, int64_t ldx, int64_t M, int64_t K,
                          float clip, int64_t n_rot, void *blocks_dev, rq_stream_t stream);
 
+/* ---- on-disk format tools (host memory, no GPU work) --------------------------------------------- */
+
+/* Replaces `pack` of the reference's converter (src/gptq.rs:210-231): N rows of K int4 codes (as int8, -8..7) and
+ * one scale per row -> N * K/256 blocks with d = scale, sum = the row's code sum (legacy header, multiplier 1),
+ * pad[0] = K, pad[1] = 0. */
+int rq_w4a4_pack(const int8_t *codes, const float *scales, int64_t N, int64_t K, void *blocks);
+
+/* Replaces `pack_groups` (src/gptq.rs:193-207): as rq_w4a4_pack, then sum = 1<<30 | k (mults_per_block = 1) or
+ * 3<<29 | k0 | k1<<4 | k2<<8 | k3<<12 (mults_per_block = 4); mults holds mults_per_block bytes per block. */
+int rq_w4a4_pack_groups(const int8_t *codes, const float *units, const uint8_t *mults, int mults_per_block,
+                        int64_t N, int64_t K, void *blocks);
+
+/* Replaces the block loop of `ruquant setclip` (src/convert.rs:876-878): activation clip into pad[1] of every
+ * block; 0 clears it (back to 1, or the environment). */
+void rq_w4a4_set_clip(void *blocks, int64_t n_blocks, float clip);
+
+/* Replaces `set_rot_len` (src/convert.rs:99-101): Hadamard length into pad[0] of every block. */
+void rq_w4a4_set_rot_len(void *blocks, int64_t n_blocks, int32_t n);
+
+/* Replaces dequantize_row_w4a4 (P:2738-2742), the type's to_float: y = code * ((float) k_g * d) for N rows of K. */
+int rq_w4a4_dequantize_rows(const void *blocks, int64_t N, int64_t K, float *out);
+
 /* Library version, for the host binding to check. */
 int rq_w4a4_abi_version(void);
 

@@ -5,9 +5,10 @@
  * Pinned against: the known answers of the compiled reference (hashes of Hadamard outputs, activation
  * blocks and vec_dot results at K = 256 .. 17408, three clips), closed forms (all-zero row,
  * non-negative row), H H^T = I, the dense +-1 matrix product on small integers, and brute-force integer
- * dot products. The weight-side quantizer (rqo_quantize_row_w*) has no reference-made vector:
- * PARITY UNPINNED for that function; it is only used to build adversarial test weights, never as an
- * expected value.
+ * dot products. The W4A4 weight dequantizer is pinned by the assertion the reference's own test makes about
+ * ggml's to_float (src/gptq.rs:313-319: code * (multiplier * unit), both multiplier encodings). The weight-side
+ * quantizer (rqo_quantize_row_w*) has no reference-made vector: PARITY UNPINNED for that function; it is only
+ * used to build adversarial test weights, never as an expected value.
  *
  * Build: gcc -O3 -ffp-contract=off (no -ffast-math).
  */

@@ -101,7 +101,6 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
         if ((reinterpret_cast<uintptr_t>(prepared[i]) & 255) != 0) return RQ_E_WORKSPACE;
         if (N[i] > Nmax) Nmax = N[i];
     }
-    if (env().act_group != 64) return RQ_E_UNSUPPORTED;
     if (!(clip > 0.0f) || !isfinite(clip)) return RQ_E_ARGUMENT;
     if (ldx < K || (ldx * 4) % 16 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0) return RQ_E_ARGUMENT;
     int p, m;
@@ -112,7 +111,10 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     if (ws_bytes < W.bytes || (reinterpret_cast<uintptr_t>(ws) & 255) != 0) return RQ_E_WORKSPACE;
     uint8_t *wsb = reinterpret_cast<uint8_t *>(ws);
 
-    const Path path = path_of(M);
+    // Activation groups of 128 / 256 (RQ_ACT_GROUP) change where the per-group floor falls; only the narrow-tile
+    // MFMA kernel folds at that granularity, so every token count takes it (a format variant, not a tuned path).
+    const int G = env().act_group;
+    const Path path = G != 64 ? kPathGemm : path_of(M);
     const bool gemm = path != kPathGemv;   // the int8 digit planes feed both MFMA kernels
     RotQuantArgs q;
     memset(&q, 0, sizeof q);
@@ -126,6 +128,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     q.m = m;
     q.scale = 1.0f / sqrtf((float) q.n_rot);
     q.clip = clip;
+    q.G = G;
     // Skinny batches with a long Paley stage: one workgroup per token would leave most of the chip idle for tens of
     // microseconds, so the rotation runs spread over workgroups (ranges out) and a second small kernel quantizes.
     const bool two_step = path == kPathSkinny && q.rotate && p >= 44 && (m & 63) == 0;
@@ -193,6 +196,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             g.ldy = ldy[i];
             g.M = (int) M;
             g.Mp = (int) W.Mp;
+            g.groups_per_fold = G / kGroup;
             e = launch_gemm(g, stream);
             if (e != hipSuccess) return (int) e;
         } else {
@@ -239,7 +243,6 @@ int rq_w4a4_supported(int type, int64_t K, int64_t N, int64_t M, int64_t ldx_byt
     if (!shape_ok(type, K, N, M)) return 0;
     if (ldx_bytes % 16 != 0 || ldx_bytes < K * 4) return 0;
     if (ldy_bytes % 4 != 0 || ldy_bytes < N * 4) return 0;
-    if (env().act_group != 64) return 0;
     if (type == RQ_TYPE_W4A4H) {
         int p, m;
         if (!hadamard_factor(K, p, m)) return 0;  // the whole-row rotation must exist (reference line 1986)
@@ -328,6 +331,7 @@ int rq_w4a4_hadamard(const float *x_dev, int64_t ldx, int64_t M, int64_t K, int6
     q.m = m;
     q.scale = 1.0f / sqrtf((float) n_rot);
     q.clip = 1.0f;
+    q.G = kGroup;
     q.mode = kActRotateOnly;
     q.out_f32 = out_dev;
     q.ldo = ldo;
@@ -339,7 +343,6 @@ int rq_w4a4_quantize_act(int type, const float *x_dev, int64_t ldx, int64_t M, i
     if (!x_dev || !blocks_dev) return RQ_E_ARGUMENT;
     if (type != RQ_TYPE_A4 && type != RQ_TYPE_A4H) return RQ_E_UNSUPPORTED;
     if (K <= 0 || K % RQ_BLOCK_CODES != 0 || K > RQ_MAX_K || M < 0) return RQ_E_UNSUPPORTED;
-    if (env().act_group != 64) return RQ_E_UNSUPPORTED;
     if (!(clip > 0.0f) || !isfinite(clip)) return RQ_E_ARGUMENT;
     if (ldx < K || (ldx * 4) % 16 != 0 || (reinterpret_cast<uintptr_t>(x_dev) & 15) != 0) return RQ_E_ARGUMENT;
     if ((reinterpret_cast<uintptr_t>(blocks_dev) & 15) != 0) return RQ_E_ARGUMENT;
@@ -359,6 +362,7 @@ int rq_w4a4_quantize_act(int type, const float *x_dev, int64_t ldx, int64_t M, i
     q.m = m;
     q.scale = 1.0f / sqrtf((float) q.n_rot);
     q.clip = clip;
+    q.G = env().act_group;
     q.mode = kActBlocks;
     q.blocks = blocks_dev;
     q.len_field = (int32_t) (had ? n_rot : K);

@@ -122,6 +122,7 @@ struct RotQuantArgs {
     int          n_rot, p, m;
     float        scale;  // 1 / sqrtf(n_rot), computed on the host exactly as the reference does
     float        clip;
+    int          G;      // activation group: 64, or 128 / 256 under RQ_ACT_GROUP (one-workgroup kernel, blocks and digits)
     int          mode;
     // outputs
     float       *out_f32;  int64_t ldo;   // kActRotateOnly, kActStats (may be null when rotate == 0)
@@ -169,6 +170,7 @@ struct GemmArgs {
     float          *y;
     int64_t         ldy;
     int             M, Mp;
+    int             groups_per_fold;   // 1; 2 or 4 when the activation groups are 128 or 256 wide
 };
 hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
 

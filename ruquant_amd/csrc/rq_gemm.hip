@@ -68,6 +68,7 @@ struct Ctx {
     size_t a_cell, a_step;
     int wave, wr, wc, l16, quad;   // wc: token half (wide) or K half (narrow)
     int ng;
+    int gs;                        // 64-wide groups per activation group (narrow tiles only): 1, 2 or 4
 };
 
 // One LDS-direct load: 64 lanes x 16 bytes from the lanes' global addresses to 1 KiB of LDS starting at `lds`
@@ -245,6 +246,67 @@ __device__ __forceinline__ void compute_pair(const Ctx &c, const Stage &sa, cons
     }
 }
 
+// Narrow tiles with activation groups of 128 or 256 (RQ_ACT_GROUP): the quantizer's multiplier and zero point, and
+// with them the floor of the fold, cover gs = 2 or 4 consecutive groups of 64. A pair of steps holds groups
+// 4i .. 4i+3 (two per stage). gs = 2: wave column wc owns the two groups of stage wc. gs = 4: the four groups are one
+// unit; the wave columns take such units alternately. The digit sums of a unit chain through the MFMA accumulator
+// and are floored once. A format variant: correct first, no software pipeline.
+template <bool HASK>
+__device__ __forceinline__ void compute_units(const Ctx &c, const Stage &cur0, const Stage &cur1,
+                                              const uint8_t *__restrict__ k_src, int st, v4i (&hi)[4][2],
+                                              int32_t (&lo)[4][2][4]) {
+    int g0;
+    if (c.gs == 2) {
+        g0 = 2 * (st + c.wc);
+    } else {
+        if (((st >> 1) & 1) != c.wc) return;
+        g0 = 2 * st;
+    }
+    if (g0 >= c.ng) return;   // ng is a multiple of gs: a unit is whole or absent (wave-uniform)
+    const int a_off = (c.wr * 2 + (c.quad >> 1)) * 64 + c.l16;
+    const int b_off = 1024 + c.quad * kBTn + c.l16;
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+        int kk[4] = { 1, 1, 1, 1 };
+        if (HASK) {
+            // the multiplier of the unit's first 64 inputs, as RQ_W_MULT_G(sum, sg << (2 - lsub)) picks it
+            // (reference patch line 171)
+            const uint32_t k4 = *reinterpret_cast<const uint32_t *>(k_src + (size_t) g0 * kPanelRows + 16 * rt);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) kk[i] = (k4 >> (8 * i)) & 0xFF;
+        }
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) {
+            v4i S = v4i{ 0, 0, 0, 0 };
+            v4i H = HASK ? v4i{ 0, 0, 0, 0 } : hi[rt][ct];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (j < c.gs) {
+                    const Stage &sg = c.gs == 2 ? (c.wc ? cur1 : cur0) : (j < 2 ? cur0 : cur1);
+                    const int gi = j & 1;   // group within the stage
+                    const uint2 pk = *(reinterpret_cast<const uint2 *>(&sg.cell[gi * 512 + a_off + 16 * rt]) + (c.quad & 1));
+                    int e0, o0, e1, o1;
+                    widen(pk.x, e0, o0);
+                    widen(pk.y, e1, o1);
+                    const v4i A = v4i{ e0, o0, e1, o1 };
+                    const v4i Blo = as_v4i(sg.cell[b_off + gi * 256 + 16 * ct]);
+                    const v4i Bhi = as_v4i(sg.cell[b_off + gi * 256 + 4 * kBTn + 16 * ct]);
+                    S = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, Blo, S, 0, 0, 0);
+                    H = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, Bhi, H, 0, 0, 0);
+                }
+            }
+            if (!HASK) {
+                hi[rt][ct] = H;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) lo[rt][ct][i] += S[i] >> 8;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) lo[rt][ct][i] += (kk[i] * ((H[i] << 6) + S[i])) >> 8;
+            }
+        }
+    }
+}
+
 // One pair of steps: wait for their operands, meet the other wavefronts, refill the two stages that were just
 // released, compute. At the wait, the loads this thread has issued after this pair's are those of the next pair.
 template <bool HASK, bool NARROW>
@@ -256,6 +318,12 @@ __device__ __forceinline__ void pair_step(const Ctx &c, const Stage &cur0, const
     asm volatile("" ::: "memory");
     fetch<NARROW>(c, refill0, st + 4);
     fetch<NARROW>(c, refill1, st + 5);
+    if constexpr (NARROW) {
+        if (c.gs > 1) {
+            compute_units<HASK>(c, cur0, cur1, k_src, st, hi, lo);
+            return;
+        }
+    }
     if constexpr (!HASK) {
         // narrow tiles: the wavefront's second group exists if 2 (st + 1) + wc < ng
         const bool both = NARROW ? 2 * (st + 1) + c.wc < c.ng : st + 1 < n_steps;
@@ -292,7 +360,7 @@ __global__ void __launch_bounds__(kThreads)
 rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                const int32_t *__restrict__ flags, const uint4 *__restrict__ act8, const float *__restrict__ u,
                float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng, int n_panels, int n_tok_tiles,
-               int first_tile, int n_tiles) {
+               int first_tile, int n_tiles, int gs) {
     // one array per stage: the compiler tracks LDS-direct loads per destination object
     __shared__ Stage s0;
     __shared__ Stage s1;
@@ -329,6 +397,7 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     c.l16 = tid & 15;
     c.quad = (tid & 63) >> 4;
     c.ng = ng;
+    c.gs = gs;
     // weights: thread tid moves cell tid of a group's 512 (panel = tid >> 7, half = (tid >> 6) & 1, row = tid & 63);
     // panels past the tensor read panel n_panels - 1 again (their outputs are never stored)
     const int w_panel = min(panel0 + (tid >> 7), n_panels - 1);
@@ -440,7 +509,7 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     const int kCUs = 256;
     int n_wide = n_tiles / kCUs * kCUs;          // whole rounds of the chip
     if (force == 0) n_wide = n_tiles;
-    if (force == 1) n_wide = 0;
+    if (force == 1 || a.groups_per_fold > 1) n_wide = 0;   // wider activation groups: narrow tiles only
     const uint4 *codes = reinterpret_cast<const uint4 *>(p + a.L.off_codes);
     const float *s_w = reinterpret_cast<const float *>(p + a.L.off_sw);
     const int32_t *flags = reinterpret_cast<const int32_t *>(p + a.L.off_flags);
@@ -448,13 +517,13 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     if (n_wide > 0) {
         hipLaunchKernelGGL(rq_gemm_kernel<false>, dim3(n_wide), dim3(kThreads), 0, stream, codes, s_w,
                            p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
-                           n_tok_tiles, 0, n_wide);
+                           n_tok_tiles, 0, n_wide, 1);
     }
     if (n_wide < n_tiles) {
         const int rest = n_tiles - n_wide;
         hipLaunchKernelGGL(rq_gemm_kernel<true>, dim3((rest + 7) / 8 * 32), dim3(kThreads), 0, stream, codes, s_w,
                            p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
-                           n_tok_tiles, n_wide, n_tiles);
+                           n_tok_tiles, n_wide, n_tiles, a.groups_per_fold);
     }
     return hipGetLastError();
 }

@@ -129,7 +129,8 @@ __global__ void __launch_bounds__(kNT, SLICED ? 2 : (P >= 44 ? 4 : 6)) rq_rotate
     }
 
     // ---- group ranges [min(x,0), max(x,0)] * clip and the token's widest range (reference lines 2646-2654)
-    const int nw = K >> 3;  // code words of this token: a thread per word, 8 lanes per group of 64
+    const int nw = K >> 3;  // code words of this token: a thread per word, lpg lanes per activation group
+    const int lpg = a.G >> 3, lgl = __ffs(lpg) - 1;   // 8, 16 or 32 lanes: groups of 64, 128 or 256 (RQ_ACT_GROUP)
     float rmax = 0.0f;
     for (int w0 = 0; w0 < nw; w0 += kNT) {
         const int w = w0 + tid;
@@ -142,16 +143,15 @@ __global__ void __launch_bounds__(kNT, SLICED ? 2 : (P >= 44 ? 4 : 6)) rq_rotate
             mn = fminf(fminf(fminf(fminf(mn, v0.x), fminf(v0.y, v0.z)), fminf(fminf(v0.w, v1.x), fminf(v1.y, v1.z))), v1.w);
             mx = fmaxf(fmaxf(fmaxf(fmaxf(mx, v0.x), fmaxf(v0.y, v0.z)), fmaxf(fmaxf(v0.w, v1.x), fmaxf(v1.y, v1.z))), v1.w);
         }
-#pragma unroll
-        for (int off = 1; off < 8; off <<= 1) {
+        for (int off = 1; off < lpg; off <<= 1) {
             mn = fminf(mn, __shfl_xor(mn, off, 64));
             mx = fmaxf(mx, __shfl_xor(mx, off, 64));
         }
         const float lo = mn * a.clip, hi = mx * a.clip;
         if (on) {
-            if ((tid & 7) == 0) {
-                g_lo[w >> 3] = lo;
-                g_hi[w >> 3] = hi;
+            if ((tid & (lpg - 1)) == 0) {
+                g_lo[w >> lgl] = lo;
+                g_hi[w >> lgl] = hi;
             }
             rmax = fmaxf(rmax, hi - lo);
         }
@@ -190,8 +190,8 @@ __global__ void __launch_bounds__(kNT, SLICED ? 2 : (P >= 44 ? 4 : 6)) rq_rotate
         const int w = w0 + tid;
         const bool on = w < nw;
         const int wc = on ? w : 0;
-        const int g = wc >> 3;
-        const float lo = g_lo[g], hi = g_hi[g];
+        const int g = wc >> 3;                     // 64-wide group: where the digits go
+        const float lo = g_lo[wc >> lgl], hi = g_hi[wc >> lgl];
         const int mg = (int) fminf(fmaxf(ceilf(((hi - lo) * 255.0f) / R), 1.0f), 255.0f);
         const float inv = 1.0f / ((float) mg * u);
         const float zf = fminf(fmaxf(rintf(-lo * inv), 0.0f), 15.0f);
@@ -235,19 +235,24 @@ __global__ void __launch_bounds__(kNT, SLICED ? 2 : (P >= 44 ? 4 : 6)) rq_rotate
         for (int j = 0; j < 8; ++j) word |= (uint32_t) ((q[j] - 8) & 0xF) << (4 * j);
 
         {  // kActBlocks: the reference's A4 / A4H storage (reference lines 2656-2661, 2667-2669)
-            const int base = tid & 32;  // lanes base, base+8, base+16, base+24 hold the block's four groups
+            const int base = tid & 32;  // lanes base, base + lpg, ... hold the block's 4, 2 or 1 groups
             uint32_t zs = 0, ms = 0;
 #pragma unroll
             for (int sg = 0; sg < 4; ++sg) {
-                zs |= (uint32_t) __shfl(z, base + 8 * sg, 64) << (4 * sg);
-                ms |= (uint32_t) __shfl(mg, base + 8 * sg, 64) << (8 * sg);
+                const uint32_t zv = (uint32_t) __shfl(z, base + ((lpg * sg) & 31), 64);
+                const uint32_t mv = (uint32_t) __shfl(mg, base + ((lpg * sg) & 31), 64);
+                if (sg * lpg < 32) {
+                    zs |= zv << (4 * sg);
+                    ms |= mv << (8 * sg);
+                }
             }
+            const uint32_t lsub = a.G == 64 ? 2u : a.G == 128 ? 1u : 0u;
             if (on) {
                 rq_block_w4a4 *blk = reinterpret_cast<rq_block_w4a4 *>(a.blocks) + (size_t) t * (K / RQ_BLOCK_CODES) + (w >> 5);
                 blk->qs[w & 31] = word;
                 if ((w & 31) == 0) {
                     blk->d = u;
-                    blk->sum = (int32_t) ((2u << 16) | zs);
+                    blk->sum = (int32_t) ((lsub << 16) | zs);
                     blk->pad[0] = (int32_t) ms;
                     blk->pad[1] = a.len_field;
                 }

@@ -51,6 +51,12 @@ PROTOTYPES = {
                                              ctypes.c_void_p]),
     "rq_w4a4_hadamard": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                         ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
+    "rq_w4a4_pack": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),
+    "rq_w4a4_pack_groups": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                           ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),
+    "rq_w4a4_set_clip": (None, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_float]),
+    "rq_w4a4_set_rot_len": (None, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32]),
+    "rq_w4a4_dequantize_rows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),
     "rq_w4a4_quantize_act": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
                                             ctypes.c_int64, ctypes.c_float, ctypes.c_int64, ctypes.c_void_p,
                                             ctypes.c_void_p]),

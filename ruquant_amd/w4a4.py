@@ -158,3 +158,53 @@ def quantize_act(x, clip, hadamard_=False, n_rot=None):
                                     M, K, clip, (n_rot or K) if hadamard_ else 0, out.data_ptr(), _stream_ptr())
     _check(rc, "rq_w4a4_quantize_act")
     return out.cpu().numpy().view(BLOCK_DTYPE).reshape(M, K // 256)
+
+
+# ---- on-disk format tools (host memory; the converter side of the reference) ----------------------------------
+
+def pack(codes, scales):
+    """int4 codes [N, K] (int8, -8..7) and one scale per row -> blocks [N, K/256] (src/gptq.rs:210-231 `pack`)."""
+    codes = np.ascontiguousarray(codes, dtype=np.int8)
+    scales = np.ascontiguousarray(scales, dtype=np.float32)
+    N, K = codes.shape
+    assert scales.shape == (N,)
+    out = np.zeros((N, K // 256), dtype=BLOCK_DTYPE)
+    _check(load_library().rq_w4a4_pack(codes.ctypes.data, scales.ctypes.data, N, K, out.ctypes.data), "rq_w4a4_pack")
+    return out
+
+
+def pack_groups(codes, units, mults):
+    """As pack, with integer weight multipliers: mults [N, K/256] (per block) or [N, K/64] (per 64 inputs)
+    (src/gptq.rs:193-207 `pack_groups`)."""
+    codes = np.ascontiguousarray(codes, dtype=np.int8)
+    units = np.ascontiguousarray(units, dtype=np.float32)
+    mults = np.ascontiguousarray(mults, dtype=np.uint8)
+    N, K = codes.shape
+    per = mults.shape[1] // (K // 256)
+    assert mults.shape == (N, per * (K // 256)) and per in (1, 4)
+    out = np.zeros((N, K // 256), dtype=BLOCK_DTYPE)
+    _check(load_library().rq_w4a4_pack_groups(codes.ctypes.data, units.ctypes.data, mults.ctypes.data, per, N, K,
+                                              out.ctypes.data), "rq_w4a4_pack_groups")
+    return out
+
+
+def set_clip(blocks, clip):
+    """Activation clip into pad[1] of every block, in place (`ruquant setclip`, src/convert.rs:876-878)."""
+    assert blocks.dtype == BLOCK_DTYPE and blocks.flags.c_contiguous
+    load_library().rq_w4a4_set_clip(blocks.ctypes.data, blocks.size, float(clip))
+
+
+def set_rot_len(blocks, n):
+    """Hadamard length into pad[0] of every block, in place (src/convert.rs:99-101 `set_rot_len`)."""
+    assert blocks.dtype == BLOCK_DTYPE and blocks.flags.c_contiguous
+    load_library().rq_w4a4_set_rot_len(blocks.ctypes.data, blocks.size, int(n))
+
+
+def dequantize_rows(blocks):
+    """The type's to_float for W4A4 weights: code * (multiplier * d) (patch lines 2738-2742). Returns [N, K] fp32."""
+    assert blocks.dtype == BLOCK_DTYPE and blocks.ndim == 2 and blocks.flags.c_contiguous
+    N, nb = blocks.shape
+    out = np.empty((N, nb * 256), dtype=np.float32)
+    _check(load_library().rq_w4a4_dequantize_rows(blocks.ctypes.data, N, nb * 256, out.ctypes.data),
+           "rq_w4a4_dequantize_rows")
+    return out

@@ -166,6 +166,25 @@ def test_mul_mat_block_diagonal_rotation(oracle):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
+def test_converter_tools_feed_the_op(oracle):
+    """Blocks built by the format tools (pack_groups, set_clip, set_rot_len), as the reference's converter writes a
+    tensor, run through the op: header clip and rotation length are what the kernels use."""
+    N, K, M, type_ = 192, 2048, 5, rq.TYPE_W4A4H
+    rng = np.random.default_rng(11)
+    codes = rng.integers(-8, 8, size=(N, K), dtype=np.int8)
+    units = np.abs(rng.normal(0.02, 0.005, size=N)).astype(np.float32)
+    mults = rng.integers(1, 16, size=(N, K // 64), dtype=np.uint8)
+    blocks = rq.pack_groups(codes, units, mults)
+    rq.set_clip(blocks, 0.8)
+    rq.set_rot_len(blocks, 512)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    assert W.clip == np.float32(0.8) and W.n_rot == 512
+    x = synth.activations("student_t4", M, K, 7)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, np.float32(0.8), n_rot=512)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
 def test_mul_mat_strided_input_and_output(oracle):
     N, K, M, type_ = 320, 1536, 6, rq.TYPE_W4A4
     blocks, wf = adversarial_weights(oracle, N, K, type_)
