@@ -352,15 +352,15 @@ __device__ __forceinline__ void gemm_body(const Ctx &c, Stage &s0, Stage &s1, St
 }
 
 // Wide tiles (256 rows x 128 tokens) are the efficient shape, but a launch of T of them keeps the chip busy for
-// ceil(T / 256) rounds. So the first floor(T / 256) * 256 tiles run wide, and the rest (`first_tile` onwards) run as
-// narrow tiles: the same 256 rows x 32 tokens, with the two wavefront columns taking alternate groups of K instead of
+// ceil(T / 256) rounds. So only whole rounds (or none, or all: see launch_gemm) run wide, and the rest (`first_tile`
+// onwards) run as narrow tiles: the same 256 rows x 32 tokens, with the two wavefront columns taking alternate groups of K instead of
 // token halves and meeting in LDS at the end. Four times as many workgroups of a quarter of the work each.
 template <bool NARROW>
 __global__ void __launch_bounds__(kThreads)
 rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                const int32_t *__restrict__ flags, const uint4 *__restrict__ act8, const float *__restrict__ u,
                float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng, int n_panels, int n_tok_tiles,
-               int first_tile, int n_tiles, int gs) {
+               int first_tile, int n_tiles, int gs, int live_last) {
     // one array per stage: the compiler tracks LDS-direct loads per destination object
     __shared__ Stage s0;
     __shared__ Stage s1;
@@ -372,23 +372,26 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
 
     // Workgroups go to the eight XCDs round robin. Wide: give every XCD a contiguous run of row tiles with the token
     // tiles running fastest, so the workgroups resident on one XCD share weight and activation tiles in its L2.
-    // Narrow: the four token quarters of a tile sit 8 apart in dispatch order (same XCD, close in time).
-    int v, t0;
+    int row_tile, t0;
     if (!NARROW) {
-        v = blockIdx.x;
+        int v = blockIdx.x;
         const int per_xcd = n_tiles / 8;
         if (v < per_xcd * 8) v = (v & 7) * per_xcd + (v >> 3);
-        t0 = 0;
+        row_tile = v / n_tok_tiles;
+        t0 = (v - row_tile * n_tok_tiles) * kBT;
     } else {
-        const int b = blockIdx.x;
-        v = first_tile + (b >> 5) * 8 + (b & 7);
-        t0 = ((b >> 3) & 3) * kBTn;
-        if (v >= n_tiles) return;
+        // Narrow workgroups cover whole row tiles from `first_tile / n_tok_tiles` on; only token quarters that hold
+        // tokens are enumerated (an empty workgroup would still take a slot of the round-robin dispatch). Each XCD
+        // gets a contiguous run, so the quarters of one row tile share its weights in one L2.
+        int b = blockIdx.x;
+        const int per_xcd = n_tiles / 8;          // here: number of narrow workgroups
+        if (b < per_xcd * 8) b = (b & 7) * per_xcd + (b >> 3);
+        const int per_row = 4 * (n_tok_tiles - 1) + live_last;
+        const int r = b / per_row, slot = b - r * per_row;
+        row_tile = first_tile / n_tok_tiles + r;
+        t0 = slot * kBTn;                          // quarters are consecutive in token order
     }
-    const int row_tile = v / n_tok_tiles, tok_tile = v - row_tile * n_tok_tiles;
     const int panel0 = row_tile * 4;
-    t0 += tok_tile * kBT;
-
     const int tid = threadIdx.x;
     Ctx c;
     c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -506,8 +509,20 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     const int n_tok_tiles = a.Mp / kBT;
     const int n_tiles = n_row_tiles * n_tok_tiles;
     static const int force = getenv("RQ_GEMM_NARROW") ? atoi(getenv("RQ_GEMM_NARROW")) : -1;   // 0: never, 1: always
+    // How many tiles run wide. A round of 256 wide tiles takes about 2.6 times a round of 256 narrow ones (a
+    // quarter of the work each, at two thirds of the efficiency); rounds are whole. Candidates: all narrow, whole
+    // wide rounds (in whole row tiles) with a narrow tail, all wide.
     const int kCUs = 256;
-    int n_wide = n_tiles / kCUs * kCUs;          // whole rounds of the chip
+    const int live_last = ((a.M + kBTn - 1) / kBTn + 3) % 4 + 1;     // token quarters of the last tile that hold tokens
+    const int per_row = 4 * (n_tok_tiles - 1) + live_last;           // narrow workgroups per row tile
+    auto cost = [&](int nw) {                                        // nw: a multiple of n_tok_tiles (whole row tiles)
+        const int64_t nn = (int64_t) (n_row_tiles - nw / n_tok_tiles) * per_row;
+        return 2.6 * ((nw + kCUs - 1) / kCUs) + 1.0 * ((nn + kCUs - 1) / kCUs);
+    };
+    int n_wide = 0;
+    const int whole = n_tiles / kCUs * kCUs / n_tok_tiles * n_tok_tiles;
+    if (cost(whole) < cost(n_wide)) n_wide = whole;
+    if (cost(n_tiles) < cost(n_wide)) n_wide = n_tiles;
     if (force == 0) n_wide = n_tiles;
     if (force == 1 || a.groups_per_fold > 1) n_wide = 0;   // wider activation groups: narrow tiles only
     const uint4 *codes = reinterpret_cast<const uint4 *>(p + a.L.off_codes);
@@ -517,13 +532,13 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     if (n_wide > 0) {
         hipLaunchKernelGGL(rq_gemm_kernel<false>, dim3(n_wide), dim3(kThreads), 0, stream, codes, s_w,
                            p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
-                           n_tok_tiles, 0, n_wide, 1);
+                           n_tok_tiles, 0, n_wide, 1, 4);
     }
     if (n_wide < n_tiles) {
-        const int rest = n_tiles - n_wide;
-        hipLaunchKernelGGL(rq_gemm_kernel<true>, dim3((rest + 7) / 8 * 32), dim3(kThreads), 0, stream, codes, s_w,
+        const int n_blocks = (n_row_tiles - n_wide / n_tok_tiles) * per_row;
+        hipLaunchKernelGGL(rq_gemm_kernel<true>, dim3(n_blocks), dim3(kThreads), 0, stream, codes, s_w,
                            p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
-                           n_tok_tiles, n_wide, n_tiles, a.groups_per_fold);
+                           n_tok_tiles, n_wide, n_blocks, a.groups_per_fold, live_last);
     }
     return hipGetLastError();
 }
