@@ -4,7 +4,8 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "librq_w4a4.so")
+# RQ_LIB_PATH points the binding at another build of the same ABI (A/B measurements)
+LIB_PATH = os.environ.get("RQ_LIB_PATH") or os.path.join(_HERE, "lib", "librq_w4a4.so")
 CSRC = os.path.join(_HERE, "csrc")
 
 
