@@ -279,6 +279,10 @@ int rq_w4a4_prepare(const void *w_blocks_dev, int64_t K, int64_t N, void *prepar
     const PreparedLayout L = prepared_layout(K, N);
     if (prepared_bytes < L.bytes || (reinterpret_cast<uintptr_t>(prepared_dev) & 255) != 0) return RQ_E_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(w_blocks_dev) & 15) != 0) return RQ_E_ARGUMENT;
+    // first use of a weight on this device: also the place for set-up that must not happen under graph capture
+    hipError_t e = init_rotate_quant_kernels();
+    if (e == hipSuccess) e = init_rotate_slab_kernels();
+    if (e != hipSuccess) return (int) e;
     return (int) launch_prepare(w_blocks_dev, L, reinterpret_cast<uint8_t *>(prepared_dev), (hipStream_t) stream);
 }
 

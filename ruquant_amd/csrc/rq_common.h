@@ -144,6 +144,10 @@ hipError_t launch_rotate_quant(const RotQuantArgs &a, hipStream_t stream);
 // Activation side of the GEMV path: like launch_rotate_quant with mode kActStats, but spreads one token over
 // several workgroups when the rotation allows it (decode latency).
 hipError_t launch_rotate_stats(const RotQuantArgs &a, hipStream_t stream);
+// per-device set-up of the activation kernels (their dynamic LDS limit); done at first use of a weight, which the
+// caller keeps outside graph capture
+hipError_t init_rotate_quant_kernels();
+hipError_t init_rotate_slab_kernels();
 // digit planes (kActI8 form) from the outputs of launch_rotate_stats: rows in out_f32, ranges in lohi / rpart
 hipError_t launch_quantize_digits(const RotQuantArgs &a, hipStream_t stream);
 

@@ -168,11 +168,16 @@ __global__ void __launch_bounds__(kRT) rq_quantize_digits_kernel(const RotQuantA
 }
 
 template <int P>
+hipError_t allow_big_lds() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_rotate_slab_kernel<P>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
+}
+
+template <int P>
 hipError_t launch_slab(const RotQuantArgs &a, hipStream_t stream) {
-    static bool attr_set = false;
+    static bool attr_set = false;   // calls that never went through rq_w4a4_prepare on this device
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_rotate_slab_kernel<P>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
+        hipError_t e = allow_big_lds<P>();
         if (e != hipSuccess) return e;
         attr_set = true;
     }
@@ -192,6 +197,14 @@ hipError_t launch_slab(const RotQuantArgs &a, hipStream_t stream) {
 }
 
 }  // namespace
+
+hipError_t init_rotate_slab_kernels() {
+    hipError_t e = allow_big_lds<1>();
+    if (e == hipSuccess) e = allow_big_lds<12>();
+    if (e == hipSuccess) e = allow_big_lds<20>();
+    if (e == hipSuccess) e = allow_big_lds<68>();
+    return e;
+}
 
 hipError_t launch_rotate_stats(const RotQuantArgs &a, hipStream_t stream) {
     // The slab kernel needs whole groups per (chunk, slab): chunks that are a multiple of 64 long. Everything else,

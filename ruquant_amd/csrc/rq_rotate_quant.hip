@@ -261,12 +261,25 @@ __global__ void __launch_bounds__(kNT, SLICED ? 2 : (P >= 44 ? 4 : 6)) rq_rotate
     }
 }
 
+// the kernels keep a whole row in dynamic LDS: raise the per-kernel limit (once per device, see init_activation_kernels)
+template <int P, bool SLICED>
+hipError_t allow_big_lds() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_rotate_quant_kernel<P, SLICED>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
+}
+
+template <int P>
+hipError_t allow_big_lds_both() {
+    hipError_t e = allow_big_lds<P, false>();
+    if (e == hipSuccess && P > 1) e = allow_big_lds<P, (P > 1)>();
+    return e;
+}
+
 template <int P, bool SLICED>
 hipError_t launch_one(const RotQuantArgs &a, size_t lds, int grid, hipStream_t stream) {
-    static bool attr_set = false;
+    static bool attr_set = false;   // calls that never went through rq_w4a4_prepare on this device
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_rotate_quant_kernel<P, SLICED>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
+        hipError_t e = allow_big_lds<P, SLICED>();
         if (e != hipSuccess) return e;
         attr_set = true;
     }
@@ -287,6 +300,20 @@ hipError_t launch_p(const RotQuantArgs &a, int grid, hipStream_t stream) {
 }
 
 }  // namespace
+
+hipError_t init_rotate_quant_kernels() {
+    hipError_t e = allow_big_lds_both<1>();
+    if (e == hipSuccess) e = allow_big_lds_both<12>();
+    if (e == hipSuccess) e = allow_big_lds_both<20>();
+    if (e == hipSuccess) e = allow_big_lds_both<44>();
+    if (e == hipSuccess) e = allow_big_lds_both<60>();
+    if (e == hipSuccess) e = allow_big_lds_both<68>();
+    if (e == hipSuccess) e = allow_big_lds_both<72>();
+    if (e == hipSuccess) e = allow_big_lds_both<84>();
+    if (e == hipSuccess) e = allow_big_lds_both<104>();
+    if (e == hipSuccess) e = allow_big_lds_both<108>();
+    return e;
+}
 
 hipError_t launch_rotate_quant(const RotQuantArgs &a, hipStream_t stream) {
     const int zero_blocks = (int) ((a.zero_ints + (int64_t) kNT * 4 - 1) / ((int64_t) kNT * 4));

@@ -294,6 +294,33 @@ def test_config5_transformer_layer_chain(oracle):
 
 # ---------------------------------------------------------------- properties that hold at any size
 
+@pytest.mark.parametrize("M", [1, 8, 16, 200])
+def test_hip_graph_replays_match_eager(oracle, M):
+    """The steady-state call is graph safe (no allocation, no synchronization, no memset nodes): capture it once,
+    replay it with fresh inputs and eager work in between, and every replay must equal the oracle."""
+    N, K, type_ = 320, 1536, rq.TYPE_W4A4H
+    blocks, wf, W = _weights(oracle, N, K, type_)
+    x = torch.zeros((M, K), dtype=torch.float32, device=DEV)
+    y = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    ws = W.workspace(M)
+    xs = [adversarial_activations(M, K, type_, wf, seed=100 + i) for i in range(3)]
+    x.copy_(torch.from_numpy(xs[0]))
+    rq.mul_mat(W, x, out=y, workspace=ws)          # warm-up outside capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        rq.mul_mat(W, x, out=y, workspace=ws)
+    for i in range(3):
+        x.copy_(torch.from_numpy(xs[i]))
+        y.fill_(-1.0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        want = oracle.mul_mat(type_, blocks, xs[i], W.clip, n_rot=K)
+        got = y.cpu().numpy()
+        assert bits_equal(got, want), "replay %d: %s" % (i, first_mismatch(got, want))
+
+
 def test_rows_are_independent_and_calls_repeatable(oracle):
     """A token's output must not depend on its neighbours or on the path taken (GEMV at M=1 vs GEMM inside M=300);
     a second call with the same workspace must reproduce the first (split-K scratch left clean)."""
