@@ -187,7 +187,7 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint
 // instructions than group by group. Software pipeline in units of one 16 x 16 tile (x two groups = 4 MFMAs): the
 // MFMAs of unit i are issued while the vector ALU folds unit i - 1.
 template <bool NARROW>
-__device__ __forceinline__ void compute_pair(const Ctx &c, const Stage &sa, const Stage &sb, bool both,
+__device__ __forceinline__ void compute_pair(const Ctx &c, const Stage &sa, const Stage &sb,
                                              v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
     constexpr int TT = NARROW ? 2 : 4;
     constexpr int kDigit = NARROW ? 4 * kBTn : 4 * kBT;   // cells between the lo and the hi plane
@@ -205,10 +205,6 @@ __device__ __forceinline__ void compute_pair(const Ctx &c, const Stage &sa, cons
         widen(pb.x, e0, o0);
         widen(pb.y, e1, o1);
         Ab[rt] = v4i{ e0, o0, e1, o1 };
-    }
-    if (!both) {   // odd group count: the last pair has one group; zero weights make the second one vanish
-#pragma unroll
-        for (int rt = 0; rt < 4; ++rt) Ab[rt] = v4i{ 0, 0, 0, 0 };
     }
     v4i Sa[2], Sb[2];
     v4i B[2][4];   // [buffer][lo a, hi a, lo b, hi b] of one token tile; the next tile's are fetched a unit ahead
@@ -325,9 +321,9 @@ __device__ __forceinline__ void pair_step(const Ctx &c, const Stage &cur0, const
         }
     }
     if constexpr (!HASK) {
-        // narrow tiles: the wavefront's second group exists if 2 (st + 1) + wc < ng
-        const bool both = NARROW ? 2 * (st + 1) + c.wc < c.ng : st + 1 < n_steps;
-        if (!NARROW || 2 * st + c.wc < c.ng) compute_pair<NARROW>(c, cur0, cur1, both, hi, lo);
+        // K is a multiple of 256, so the number of groups is a multiple of 4: a pair of steps (two groups wide, four
+        // narrow) is always whole
+        compute_pair<NARROW>(c, cur0, cur1, hi, lo);
     } else {
         compute<HASK, NARROW>(c, cur0, k_src, st, hi, lo);
         if (st + 1 < n_steps) compute<HASK, NARROW>(c, cur1, k_src, st + 1, hi, lo);
@@ -377,8 +373,19 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
         int v = blockIdx.x;
         const int per_xcd = n_tiles / 8;
         if (v < per_xcd * 8) v = (v & 7) * per_xcd + (v >> 3);
-        row_tile = v / n_tok_tiles;
-        t0 = (v - row_tile * n_tok_tiles) * kBT;
+        if (gs) {
+            // (wide tiles only: gs carries the flag) super-tiles of 8 row tiles x 4 token tiles = the 32 workgroups an
+            // XCD runs at a time: together they read 8 weight tiles and 4 activation tiles, the mix that puts the
+            // least through that XCD's L2
+            const int s = v >> 5, i = v & 31;
+            const int spr = n_tok_tiles >> 2;
+            const int sr = s / spr;
+            row_tile = sr * 8 + (i >> 2);
+            t0 = ((s - sr * spr) * 4 + (i & 3)) * kBT;
+        } else {
+            row_tile = v / n_tok_tiles;
+            t0 = (v - row_tile * n_tok_tiles) * kBT;
+        }
     } else {
         // Narrow workgroups cover whole row tiles from `first_tile / n_tok_tiles` on; only token quarters that hold
         // tokens are enumerated (an empty workgroup would still take a slot of the round-robin dispatch). Each XCD
@@ -525,6 +532,10 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     if (cost(n_tiles) < cost(n_wide)) n_wide = n_tiles;
     if (force == 0) n_wide = n_tiles;
     if (force == 1 || a.groups_per_fold > 1) n_wide = 0;   // wider activation groups: narrow tiles only
+    // the super-tile order of the wide kernel needs a wide region of whole blocks of 8 row tiles x 4 token tiles
+    static const int no_super = getenv("RQ_GEMM_SUPER") ? atoi(getenv("RQ_GEMM_SUPER")) == 0 : 0;
+    const int super_tiles = !no_super && n_wide > 0 && n_tok_tiles % 4 == 0 && n_wide % n_tok_tiles == 0 &&
+                            (n_wide / n_tok_tiles) % 8 == 0;
     const uint4 *codes = reinterpret_cast<const uint4 *>(p + a.L.off_codes);
     const float *s_w = reinterpret_cast<const float *>(p + a.L.off_sw);
     const int32_t *flags = reinterpret_cast<const int32_t *>(p + a.L.off_flags);
@@ -532,7 +543,7 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     if (n_wide > 0) {
         hipLaunchKernelGGL(rq_gemm_kernel<false>, dim3(n_wide), dim3(kThreads), 0, stream, codes, s_w,
                            p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
-                           n_tok_tiles, 0, n_wide, 1, 4);
+                           n_tok_tiles, 0, n_wide, super_tiles, 4);
     }
     if (n_wide < n_tiles) {
         const int n_blocks = (n_row_tiles - n_wide / n_tok_tiles) * per_row;
