@@ -178,7 +178,7 @@ struct GemmArgs {
 };
 hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
 
-// 9..64 tokens: MFMA arithmetic on a GEMV-shaped weight stream; same operands as the GEMM plus the split-K cells
+// up to 64 tokens: MFMA arithmetic on a GEMV-shaped weight stream; same operands as the GEMM plus the split-K cells
 struct SkinnyArgs {
     const uint8_t  *prepared;
     PreparedLayout  L;

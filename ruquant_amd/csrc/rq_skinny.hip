@@ -1,4 +1,4 @@
-// int4 x int4 product for 9..64 tokens (verify batches, short prefill chunks) on the gfx950 matrix cores.
+// int4 x int4 product for a handful to 64 tokens (wide decode batches, verify batches, short prefill chunks) on the gfx950 matrix cores.
 //
 // Still a weight stream: with so few tokens the weights are read once and the work per byte is small, so the kernel
 // is shaped like the GEMV (a workgroup = one panel of 64 rows x one slice of K, no LDS staging and no barriers in
