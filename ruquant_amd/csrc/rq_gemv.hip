@@ -256,8 +256,8 @@ hipError_t launch_t(const GemvArgs &a, int nks, hipStream_t stream) {
 
 // How many workgroups share K for one panel. The kernel is a pure stream with a latency-bound start and end, so
 // it wants many small workgroups: their starts and tails overlap and the last wave of workgroups is short. Aim for
-// about a thousand workgroups, at least a batch (kGemvWaves x kUnroll groups) each when K allows, never fewer than
-// four groups per workgroup, and never more than kMaxSlice (the slice's codes live in LDS).
+// about a thousand workgroups, at least a batch (kGemvWaves x kUnroll groups) each when K allows, at least ten groups
+// per workgroup, and never more than kMaxSlice (the slice's codes live in LDS).
 int gemv_ksplit(const PreparedLayout &L) {
     static const int forced = getenv("RQ_GEMV_KSPLIT") ? atoi(getenv("RQ_GEMV_KSPLIT")) : 0;
     int nks;
@@ -266,8 +266,11 @@ int gemv_ksplit(const PreparedLayout &L) {
     } else {
         const int by_batch = (L.ng + kGemvWaves * kUnroll - 1) / (kGemvWaves * kUnroll);
         const int by_grid = (1024 + L.n_panels - 1) / L.n_panels;
+        // more splits than ng / 10 cost more in atomics and short workgroups than they gain in parallelism (measured
+        // on 16..96 panels)
+        const int cap = L.ng / 10 > by_batch ? L.ng / 10 : by_batch;
         nks = by_batch > by_grid ? by_batch : by_grid;
-        if (nks > L.ng / 4) nks = L.ng / 4;
+        if (nks > cap) nks = cap;
     }
     const int least = (L.ng + kMaxSlice - 1) / kMaxSlice;   // ceil(ng / nks) <= kMaxSlice
     if (nks < least) nks = least;
