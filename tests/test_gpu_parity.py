@@ -154,6 +154,19 @@ def test_mul_mat_token_counts_between_gemv_and_gemm(oracle, M):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
+@pytest.mark.parametrize("type_", [rq.TYPE_W4A4, rq.TYPE_W4A4H], ids=["w4a4", "w4a4h"])
+@pytest.mark.parametrize("M", [1, 7, 70])
+def test_mul_mat_longest_row(oracle, type_, M):
+    """K = 32768, the longest row the op takes (RQ_MAX_K): one Sylvester transform of 2^15, 512 groups, all three
+    product kernels."""
+    N, K = 128, 32768
+    blocks, wf, W = _weights(oracle, N, K, type_)
+    x = adversarial_activations(M, K, type_, wf, seed=3 * M)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=max(W.n_rot, 0))
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
 def test_mul_mat_block_diagonal_rotation(oracle):
     """Hadamard length shorter than the row (pad[0] = K / 4), as ruquant convert --rot-blocks writes."""
     N, K, M, type_ = 128, 6144, 9, rq.TYPE_W4A4H
