@@ -19,7 +19,11 @@ namespace rq {
 
 namespace {
 
-constexpr int kNT = 512;  // threads per token workgroup
+// Threads per token workgroup. Small batches (the sliced variant) with a short Paley stage get 1024: there the kernel
+// is one workgroup per compute unit at most, bound by the latency of its own phases, and twice the threads halve the
+// work per phase. Long Paley stages keep their columns in registers and need the 256-register budget of 512 threads.
+template <int P, bool SLICED>
+constexpr int threads_of() { return SLICED && P < 44 ? 1024 : 512; }
 
 using namespace had;
 
@@ -27,7 +31,9 @@ template <int P, bool SLICED>
 // Registers are capped so that two workgroups (p >= 44: long columns, long rows) or three fit a compute unit: the
 // stages of one token are separated by barriers, and it is the other workgroups that keep the vector ALU busy. (The
 // sliced variant serves small batches, where occupancy is not the limit.)
-__global__ void __launch_bounds__(kNT, SLICED ? 2 : (P >= 44 ? 4 : 6)) rq_rotate_quant_kernel(const RotQuantArgs a) {
+__global__ void __launch_bounds__((threads_of<P, SLICED>()), SLICED ? (P < 44 ? 4 : 2) : (P >= 44 ? 4 : 6))
+rq_rotate_quant_kernel(const RotQuantArgs a) {
+    constexpr int kNT = threads_of<P, SLICED>();
     extern __shared__ __align__(16) float smem[];
     __shared__ float s_red[kNT / 64];
 
@@ -276,27 +282,33 @@ hipError_t allow_big_lds_both() {
 }
 
 template <int P, bool SLICED>
-hipError_t launch_one(const RotQuantArgs &a, size_t lds, int grid, hipStream_t stream) {
+hipError_t launch_one(const RotQuantArgs &a, size_t lds, hipStream_t stream) {
     static bool attr_set = false;   // calls that never went through rq_w4a4_prepare on this device
     if (!attr_set) {
         hipError_t e = allow_big_lds<P, SLICED>();
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL((rq_rotate_quant_kernel<P, SLICED>), dim3(grid), dim3(kNT), lds, stream, a);
+    constexpr int kNT = threads_of<P, SLICED>();
+    // blocks past the tokens clear the split-K cells, four ints per thread
+    RotQuantArgs b = a;
+    b.token_blocks = a.M;
+    const int grid = a.M + (int) ((a.zero_ints + (int64_t) kNT * 4 - 1) / ((int64_t) kNT * 4));
+    if (grid == 0) return hipSuccess;
+    hipLaunchKernelGGL((rq_rotate_quant_kernel<P, SLICED>), dim3(grid), dim3(kNT), lds, stream, b);
     return hipGetLastError();
 }
 
 // LDS: one padded row (two when the Paley stage is sliced over more threads) plus the group ranges. Slicing buys
 // parallelism inside a token and costs occupancy, so it is for small batches only.
 template <int P>
-hipError_t launch_p(const RotQuantArgs &a, int grid, hipStream_t stream) {
+hipError_t launch_p(const RotQuantArgs &a, hipStream_t stream) {
     const size_t row = (size_t) (a.K + (a.K >> 4) + 1) * sizeof(float);
     const size_t stats = (size_t) 2 * (a.K / kGroup + 1) * sizeof(float);
     if (P > 1 && a.M <= 64 && 2 * row + stats <= 160 * 1024 - 64) {
-        return launch_one<P, (P > 1)>(a, 2 * row + stats, grid, stream);
+        return launch_one<P, (P > 1)>(a, 2 * row + stats, stream);
     }
-    return launch_one<P, false>(a, row + stats, grid, stream);
+    return launch_one<P, false>(a, row + stats, stream);
 }
 
 }  // namespace
@@ -316,23 +328,19 @@ hipError_t init_rotate_quant_kernels() {
 }
 
 hipError_t launch_rotate_quant(const RotQuantArgs &a, hipStream_t stream) {
-    const int zero_blocks = (int) ((a.zero_ints + (int64_t) kNT * 4 - 1) / ((int64_t) kNT * 4));
-    RotQuantArgs b = a;
-    b.token_blocks = a.M;
-    const int grid = a.M + zero_blocks;
-    if (grid == 0) return hipSuccess;
+    if (a.M == 0 && a.zero_ints == 0) return hipSuccess;
     const int p = a.rotate ? a.p : 1;
     switch (p) {
-        case 1:   return launch_p<1>(b, grid, stream);
-        case 12:  return launch_p<12>(b, grid, stream);
-        case 20:  return launch_p<20>(b, grid, stream);
-        case 44:  return launch_p<44>(b, grid, stream);
-        case 60:  return launch_p<60>(b, grid, stream);
-        case 68:  return launch_p<68>(b, grid, stream);
-        case 72:  return launch_p<72>(b, grid, stream);
-        case 84:  return launch_p<84>(b, grid, stream);
-        case 104: return launch_p<104>(b, grid, stream);
-        case 108: return launch_p<108>(b, grid, stream);
+        case 1:   return launch_p<1>(a, stream);
+        case 12:  return launch_p<12>(a, stream);
+        case 20:  return launch_p<20>(a, stream);
+        case 44:  return launch_p<44>(a, stream);
+        case 60:  return launch_p<60>(a, stream);
+        case 68:  return launch_p<68>(a, stream);
+        case 72:  return launch_p<72>(a, stream);
+        case 84:  return launch_p<84>(a, stream);
+        case 104: return launch_p<104>(a, stream);
+        case 108: return launch_p<108>(a, stream);
         default:  return hipErrorInvalidValue;
     }
 }
