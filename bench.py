@@ -161,7 +161,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this operator is measured on one GPU; --gpus %d is not a configuration of this build "
-              "(the op shards along N with no exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "(the op shards along N with no exchange between GPUs)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch
