@@ -48,8 +48,12 @@ __device__ __forceinline__ void load_batch(Batch &b, const uint4 *wp, int g0, in
 #pragma unroll
     for (int k = 0; k < kUnroll; ++k) {
         const int g = min(g0 + k * kWaves, g_end - 1);  // past the end: reread the last group, contribute nothing
-        b.q[k][0] = wp[(size_t) g * 128];
-        b.q[k][1] = wp[(size_t) g * 128 + 64];
+        // weights are read once per call: non-temporal, so they do not displace the activations and ranges in L2
+        typedef unsigned v4u __attribute__((ext_vector_type(4)));
+        const v4u q0 = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(wp + (size_t) g * 128));
+        const v4u q1 = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(wp + (size_t) g * 128 + 64));
+        b.q[k][0] = make_uint4(q0.x, q0.y, q0.z, q0.w);
+        b.q[k][1] = make_uint4(q1.x, q1.y, q1.z, q1.w);
     }
 }
 

@@ -47,8 +47,14 @@ struct Frag {
 
 template <int TT>
 __device__ __forceinline__ void load_frag(Frag<TT> &f, const uint8_t *a_base, const uint4 *b_base, int g, int Mp) {
+    // weights are read once (twice with two token blocks, and then from L2 at once): non-temporal, so they do not
+    // displace the digit planes, which every workgroup re-reads
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
 #pragma unroll
-    for (int rt = 0; rt < 4; ++rt) f.a[rt] = *reinterpret_cast<const uint2 *>(a_base + (size_t) g * 2048 + rt * 256);
+    for (int rt = 0; rt < 4; ++rt) {
+        const v2u v = __builtin_nontemporal_load(reinterpret_cast<const v2u *>(a_base + (size_t) g * 2048 + rt * 256));
+        f.a[rt] = make_uint2(v.x, v.y);
+    }
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
         f.b[tt][0] = b_base[(size_t) g * 8 * Mp + 16 * tt];
