@@ -497,7 +497,10 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
                 o.y = (((float) tot[rt][ct][1] * 16.0f) * ut) * sw.y;
                 o.z = (((float) tot[rt][ct][2] * 16.0f) * ut) * sw.z;
                 o.w = (((float) tot[rt][ct][3] * 16.0f) * ut) * sw.w;
-                *reinterpret_cast<float4 *>(dst) = o;
+                // the output is written once and not read back by this launch: non-temporal, so that 4 M N bytes of y
+                // do not push weight and activation tiles out of L2
+                typedef float v4f __attribute__((ext_vector_type(4)));
+                __builtin_nontemporal_store(v4f{ o.x, o.y, o.z, o.w }, reinterpret_cast<v4f *>(dst));
             } else {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
