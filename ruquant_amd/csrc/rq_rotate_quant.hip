@@ -49,7 +49,13 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
         return;
     }
 
-    const int t = blockIdx.x;
+    // Which token. In the digit-plane layout eight consecutive tokens share a 128-byte line of every (group, digit,
+    // quarter) run, and workgroups go to the eight XCDs round robin: taken in order, the eight writers of a line
+    // would sit in eight different L2s and the line would reach memory as eight partial writes. So within blocks of
+    // 64 tokens, workgroup b takes token 8 (b % 8) + (b / 8) % 8: the writers of a line share an XCD (same b % 8)
+    // and are dispatched within 64 workgroups of each other.
+    int t = blockIdx.x;
+    if (a.mode == kActI8 && t < (a.M & ~63)) t = (t & ~63) | ((t & 7) << 3) | ((t >> 3) & 7);
     const int K = a.K;
     const int ng = K / kGroup;
     const int Kp = padi(K) + 1;                  // floats of one padded row
