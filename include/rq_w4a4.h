@@ -154,6 +154,24 @@ void rq_w4a4_set_rot_len(void *blocks, int64_t n_blocks, int32_t n);
 /* Replaces dequantize_row_w4a4 (P:2738-2742), the type's to_float: y = code * ((float) k_g * d) for N rows of K. */
 int rq_w4a4_dequantize_rows(const void *blocks, int64_t N, int64_t K, float *out);
 
+/* Replaces quantize_row_w4a4_ref / quantize_row_w4a4h_ref (P:2681-2683, P:2701-2710; the types' from_float_ref) and
+ * the row loops of quantize_w4a4 / quantize_w4a4h (P:2775-2789) for a whole tensor on the GPU: N rows of K floats at
+ * w_dev (row stride ldw floats, 16-byte aligned) -> N * K/256 blocks at blocks_dev, bit-identical to the reference's
+ * output. W4A4H rows are rotated first (x diag(H_n_rot, ...), P:2697-2699); n_rot is the reference's K / RQ_ROT_BLOCKS
+ * (P:2687-2694) and lands in pad[0]. wgroup is the reference's RQ_WGROUP switch (P:2531-2538): 0 = one scale per row
+ * from the 13-ratio clip search (P:2509-2527) and the legacy row-sum header; 256 or 64 = a scale per block or per 64
+ * inputs, stored as multipliers 1..15 of the row's unit (P:2555-2575). No allocation, no synchronization. */
+size_t rq_w4a4_quantize_weights_workspace_bytes(int type, int64_t K, int64_t N, int wgroup);
+int rq_w4a4_quantize_weights(int type, const float *w_dev, int64_t ldw, int64_t N, int64_t K, int64_t n_rot, int wgroup,
+                             void *blocks_dev, void *workspace_dev, size_t workspace_bytes, rq_stream_t stream);
+
+/* Replaces dequantize_row_w4a4 / _w4a4h / _a4 / _a4h (P:2738-2773; the types' to_float) on the GPU: rows x K/256
+ * blocks of `type` (44..47) at blocks_dev -> rows of K floats at out_dev (row stride ldo floats). The rotated types
+ * are taken back to the original basis with the transposed Hadamard of length n_rot, which the caller reads from
+ * block 0 as the reference does (pad[0] of weights, pad[1] of activations; P:2757-2763); other types ignore n_rot. */
+int rq_w4a4_dequantize(int type, const void *blocks_dev, int64_t rows, int64_t K, int64_t n_rot, float *out_dev,
+                       int64_t ldo, rq_stream_t stream);
+
 /* Library version, for the host binding to check. */
 int rq_w4a4_abi_version(void);
 

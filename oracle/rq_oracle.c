@@ -7,8 +7,12 @@
  * non-negative row), H H^T = I, the dense +-1 matrix product on small integers, and brute-force integer
  * dot products. The W4A4 weight dequantizer is pinned by the assertion the reference's own test makes about
  * ggml's to_float (src/gptq.rs:313-319: code * (multiplier * unit), both multiplier encodings). The weight-side
- * quantizer (rqo_quantize_row_w*) has no reference-made vector: PARITY UNPINNED for that function; it is only
- * used to build adversarial test weights, never as an expected value.
+ * quantizer (rqo_quantize_row_w*) has no reference-made vector; it is pinned by the reference's second statement of
+ * the same row search and code rule (int4_scale and code, src/gptq.rs:13-38, restated from the Rust text and
+ * compared bit for bit), by the minimum property of the chosen ratio in exact rational arithmetic, by what the
+ * reference's test asserts about weight groups (src/gptq.rs:303-311) and by round trips through the dequantizers
+ * (tests/test_oracle_weight_quant.py). The activation dequantizers (rqo_dequantize_row_a) are pinned only through
+ * those round-trip properties and the closed form of their one line: no reference-made value covers them.
  *
  * Build: gcc -O3 -ffp-contract=off (no -ffast-math).
  */

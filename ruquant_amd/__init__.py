@@ -9,5 +9,5 @@ from .w4a4 import (  # noqa: F401
     TYPE_W4A4, TYPE_W4A4H, TYPE_A4, TYPE_A4H, BLOCK_DTYPE,
     W4A4Weight, supported, hadamard_factor, resolve_clip, tensor_rot,
     mul_mat, mul_mat_fused, hadamard, quantize_act, RqError,
-    pack, pack_groups, set_clip, set_rot_len, dequantize_rows,
+    pack, pack_groups, set_clip, set_rot_len, dequantize_rows, quantize_weights, dequantize,
 )

@@ -37,8 +37,9 @@ constexpr PaleyTable<P> make_paley() {
     return t;
 }
 
-// outputs 4S .. 4S+3 of one column: acc = ((0 +- c0) +- c1) ... in ascending chunk order
-template <int P, int S>
+// outputs 4S .. 4S+3 of one column: acc = ((0 +- c0) +- c1) ... in ascending chunk order. TR takes the signs of the
+// transposed matrix (A[a][i] instead of A[i][a], reference line 2476): the inverse rotation of the dequantizers.
+template <int P, int S, bool TR = false>
 __device__ __forceinline__ void paley_slice(const float (&col)[P], float (&out)[4]) {
     constexpr PaleyTable<P> T = make_paley<P>();
 #pragma unroll
@@ -46,7 +47,7 @@ __device__ __forceinline__ void paley_slice(const float (&col)[P], float (&out)[
         float acc = 0.0f;
 #pragma unroll
         for (int i = 0; i < P; ++i) {
-            acc = T.neg[i][4 * S + o] ? acc - col[i] : acc + col[i];
+            acc = (TR ? T.neg[4 * S + o][i] : T.neg[i][4 * S + o]) ? acc - col[i] : acc + col[i];
         }
         out[o] = acc;
     }
@@ -62,26 +63,26 @@ __device__ __forceinline__ void paley_pick(int s, const float (&col)[P], float (
 }
 
 // all P outputs of one column, written back in place (the column is private to the calling thread)
-template <int P, int S = 0>
+template <int P, int S = 0, bool TR = false>
 __device__ __forceinline__ void paley_column(const float (&col)[P], float *dst, int stride, float scale) {
     float out[4];
-    paley_slice<P, S>(col, out);
+    paley_slice<P, S, TR>(col, out);
 #pragma unroll
     for (int o = 0; o < 4; ++o) dst[(4 * S + o) * stride] = out[o] * scale;
-    if constexpr (S + 1 < P / 4) paley_column<P, S + 1>(col, dst, stride, scale);
+    if constexpr (S + 1 < P / 4) paley_column<P, S + 1, TR>(col, dst, stride, scale);
 }
 
 // same, for chunk lengths that are not a multiple of 16 (the padded stride is then not uniform)
-template <int P, int S = 0>
+template <int P, int S = 0, bool TR = false>
 __device__ __forceinline__ void paley_column_generic(const float (&col)[P], float *buf, int b0, int m, float scale) {
     float out[4];
-    paley_slice<P, S>(col, out);
+    paley_slice<P, S, TR>(col, out);
 #pragma unroll
     for (int o = 0; o < 4; ++o) {
         const int i = b0 + (4 * S + o) * m;
         buf[i + (i >> 4)] = out[o] * scale;
     }
-    if constexpr (S + 1 < P / 4) paley_column_generic<P, S + 1>(col, buf, b0, m, scale);
+    if constexpr (S + 1 < P / 4) paley_column_generic<P, S + 1, TR>(col, buf, b0, m, scale);
 }
 
 __device__ __forceinline__ float wave_max(float v) {

@@ -58,6 +58,13 @@ PROTOTYPES = {
     "rq_w4a4_set_clip": (None, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_float]),
     "rq_w4a4_set_rot_len": (None, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32]),
     "rq_w4a4_dequantize_rows": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),
+    "rq_w4a4_quantize_weights_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int64, ctypes.c_int64,
+                                                                  ctypes.c_int]),
+    "rq_w4a4_quantize_weights": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                                ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p,
+                                                ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "rq_w4a4_dequantize": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                          ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
     "rq_w4a4_quantize_act": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
                                             ctypes.c_int64, ctypes.c_float, ctypes.c_int64, ctypes.c_void_p,
                                             ctypes.c_void_p]),

@@ -160,6 +160,46 @@ def quantize_act(x, clip, hadamard_=False, n_rot=None):
     return out.cpu().numpy().view(BLOCK_DTYPE).reshape(M, K // 256)
 
 
+def quantize_weights(w, type_, n_rot=None, wgroup=0):
+    """w[N, K] fp32 on the GPU -> [N, K/256] weight blocks (numpy, host): the type's from_float_ref for whole
+    tensors (quantize_row_w4a4_ref / quantize_row_w4a4h_ref, patch lines 2681-2710). wgroup 0 / 256 / 64 is the
+    reference's RQ_WGROUP switch; n_rot (W4A4H) its K / RQ_ROT_BLOCKS, default K."""
+    L = load_library()
+    assert w.is_cuda and w.dtype == torch.float32 and w.dim() == 2 and w.stride(1) == 1
+    N, K = w.shape
+    n_rot = int(n_rot or K)
+    nbytes = L.rq_w4a4_quantize_weights_workspace_bytes(int(type_), K, N, int(wgroup))
+    if nbytes == 0:
+        raise RqError("unsupported weight shape or group: K=%d N=%d wgroup=%d" % (K, N, wgroup))
+    ws = _device_bytes(nbytes, w.device)
+    out = torch.zeros(N * (K // 256) * 144, dtype=torch.uint8, device=w.device)
+    with torch.cuda.device(w.device):
+        rc = L.rq_w4a4_quantize_weights(int(type_), w.data_ptr(), w.stride(0) if N > 1 else K, N, K, n_rot,
+                                        int(wgroup), out.data_ptr(), ws.data_ptr(), ws.numel(), _stream_ptr())
+    _check(rc, "rq_w4a4_quantize_weights")
+    return out.cpu().numpy().view(BLOCK_DTYPE).reshape(N, K // 256)
+
+
+def dequantize(blocks, type_, n_rot=None, device="cuda:0"):
+    """[rows, K/256] blocks of any of the four types (numpy, host) -> [rows, K] fp32 on the GPU: the type's to_float
+    (dequantize_row_w4a4 / _w4a4h / _a4 / _a4h, patch lines 2738-2773). The rotation length of the rotated types
+    comes from block 0 (pad[0] of weights, pad[1] of activations) unless given."""
+    L = load_library()
+    blocks = np.ascontiguousarray(blocks)
+    assert blocks.dtype == BLOCK_DTYPE and blocks.ndim == 2
+    rows, nb = blocks.shape
+    K = nb * 256
+    if n_rot is None:
+        n_rot = int(blocks[0, 0]["pad"][0 if type_ in (TYPE_W4A4, TYPE_W4A4H) else 1]) if rows else K
+    dev = torch.device(device)
+    raw = torch.from_numpy(blocks.view(np.uint8).reshape(-1).copy()).to(dev)
+    out = torch.empty((rows, K), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = L.rq_w4a4_dequantize(int(type_), raw.data_ptr(), rows, K, int(n_rot), out.data_ptr(), K, _stream_ptr())
+    _check(rc, "rq_w4a4_dequantize")
+    return out
+
+
 # ---- on-disk format tools (host memory; the converter side of the reference) ----------------------------------
 
 def pack(codes, scales):
