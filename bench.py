@@ -11,7 +11,8 @@ Prints one JSON line. Besides the contract fields it carries
   roofline     : the product kernel alone (HIP events around back-to-back launches on the launch stream),
   cpu_baseline : the CPU oracle (a bit-identical restatement of the ggml-cpu reference path) on the host cores,
   extra        : the same measurements for the other benchmark shapes (M = 2048 prefill as TOPS against the dense
-                 int8 MFMA peak, the N = 5120 decode shapes, the K = 17408 down projection).
+                 int8 MFMA peak, the N = 5120 decode shapes, the K = 17408 down projection) and the seven matmuls of
+                 one transformer layer at 16 tokens, run in the layer's dataflow.
 """
 import argparse
 import json
@@ -116,6 +117,85 @@ class Problem:
         return bool((got.view(np.uint32) == want.view(np.uint32)).all())
 
 
+class Layer:
+    """The seven W4A4H matmuls of one transformer layer at M tokens, in the layer's dataflow: q, k, v <- x0 (one
+    fused call: the three weights share one rotation + quantization of x0); o <- q's output; gate, up <- o's output
+    (fused); down <- up's output. Clip 1.0, whole-row rotations (H20xH256, H12xH512 for o, H68xH256 for down). Two
+    sets of weights alternate so that successive layers read 341 MB of codes, more than the Infinity Cache holds."""
+
+    SHAPES = [("q", 5120, 6144), ("k", 5120, 1024), ("v", 5120, 1024), ("o", 6144, 5120), ("gate", 5120, 17408),
+              ("up", 5120, 17408), ("down", 17408, 5120)]
+
+    def __init__(self, M, seed=1, copies=2, dev="cuda:0"):
+        import torch
+        import ruquant_amd as rq
+        from ruquant_amd import synth
+        self.rq, self.torch, self.M = rq, torch, M
+        self.sets = []
+        for c in range(copies):
+            ws = {}
+            for i, (name, K, N) in enumerate(self.SHAPES):
+                blocks = synth.random_weight_blocks(N, K, seed + i, rq.TYPE_W4A4H, clip=0.0)
+                ws[name] = rq.W4A4Weight(blocks, rq.TYPE_W4A4H, dev, keep_blocks=False)
+            self.sets.append(ws)
+        self.x0 = torch.from_numpy(synth.activations("normal", M, 5120, seed)).to(dev)
+        self.out = {name: torch.empty((M, N), dtype=torch.float32, device=dev) for name, K, N in self.SHAPES}
+        L = rq.load_library()
+        self.ws = torch.empty(max(L.rq_w4a4_workspace_bytes(rq.TYPE_W4A4H, K, N, M) for _, K, N in self.SHAPES),
+                              dtype=torch.uint8, device=dev)
+        self.code_bytes = sum(K * N // 2 for _, K, N in self.SHAPES)
+        self.bytes = sum(algorithmic_bytes(K, N, M) for _, K, N in self.SHAPES)
+        self.ops = sum(2 * M * K * N for _, K, N in self.SHAPES)
+        self.i = 0
+
+    def call(self, fused=True):
+        w = self.sets[self.i % len(self.sets)]
+        self.i += 1
+        rq, o = self.rq, self.out
+        if fused:
+            rq.mul_mat_fused([w["q"], w["k"], w["v"]], self.x0, outs=[o["q"], o["k"], o["v"]], workspace=self.ws)
+        else:
+            for n in ("q", "k", "v"):
+                rq.mul_mat(w[n], self.x0, out=o[n], workspace=self.ws)
+        rq.mul_mat(w["o"], o["q"], out=o["o"], workspace=self.ws)
+        if fused:
+            rq.mul_mat_fused([w["gate"], w["up"]], o["o"], outs=[o["gate"], o["up"]], workspace=self.ws)
+        else:
+            for n in ("gate", "up"):
+                rq.mul_mat(w[n], o["o"], out=o[n], workspace=self.ws)
+        rq.mul_mat(w["down"], o["up"], out=o["down"], workspace=self.ws)
+
+    def timed(self, steps, warmup, fused=True):
+        torch = self.torch
+        for _ in range(max(warmup, 1)):
+            self.call(fused)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(steps):
+                self.call(fused)
+        g.replay()
+        torch.cuda.synchronize()
+        vals = []
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            vals.append(e0.elapsed_time(e1) / steps)
+        return sorted(vals)[len(vals) // 2]
+
+    def measure(self, steps, warmup):
+        fused_ms = self.timed(steps, warmup, True)
+        plain_ms = self.timed(steps, warmup, False)
+        return {"M": self.M, "matmuls": 7, "code_bytes": self.code_bytes, "layer_us": round(fused_ms * 1e3, 2),
+                "layer_gbs": round(self.bytes / fused_ms / 1e6, 1),
+                "layer_frac_of_hbm_peak": round(self.bytes / fused_ms / 1e6 / HBM_PEAK_GBS, 4),
+                "layer_tops": round(self.ops / fused_ms / 1e9, 2),
+                "layer_us_seven_separate_calls": round(plain_ms * 1e3, 2)}
+
+
 def cpu_baseline(oracle, prob, budget_s=12.0, max_reps=400):
     threads = min(os.cpu_count() or 1, 16)
     reps, t0 = 0, time.perf_counter()
@@ -216,6 +296,11 @@ def main():
             head = Problem(k, n, m, kind, clip, seed=3)
             steps = args.steps if m <= 64 else max(5, args.steps // 10)
             extra[name], _, _ = measure(head, steps, min(args.warmup, steps), bound)
+
+        if not want or "layer_m16" in want:
+            head = None
+            torch.cuda.empty_cache()
+            extra["layer_m16"] = Layer(16).measure(max(5, args.steps // 4), 3)
 
     line = {
         "metric": "w4a4h_matmul_gbps_m1", "value": round(b / op_ms / 1e6, 1), "unit": "GB/s",

@@ -190,7 +190,11 @@ struct SkinnyArgs {
     int32_t        *tot;    // split-K cells [M][n_panels * 64], 64 bits each
 };
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream);
-int skinny_ksplit(const PreparedLayout &L, int M);
+struct SkinnyPlan {
+    int main_panels;   // leading panels that run as one whole-K workgroup each
+    int tail_split;    // K slices (workgroups) per remaining panel
+};
+SkinnyPlan skinny_plan(const PreparedLayout &L, int M);
 
 hipError_t launch_prepare(const void *blocks, const PreparedLayout &L, uint8_t *prepared, hipStream_t stream);
 

@@ -148,8 +148,9 @@ template <int TT>
 __global__ void __launch_bounds__(kThreads, TT == 1 ? 4 : 2)   // wavefronts per SIMD: two workgroups per CU at TT = 1
 rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                  const int32_t *__restrict__ flags, const uint4 *__restrict__ act8, const float *__restrict__ u,
-                 float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng, int n_panels, int nz,
-                 unsigned long long *__restrict__ cells, int n_rows_pad, int slice_base, int slice_extra) {
+                 float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng, int n_units, int nz,
+                 unsigned long long *__restrict__ cells, int n_rows_pad, int main_panels, int tail_split,
+                 int slice_base, int slice_extra) {
     constexpr int kTok = TT * 16;
     constexpr int kStride = kTok + 1;             // padded: the epilogue reads a column of this array
     __shared__ int32_t s_tot[64 * kStride];
@@ -161,13 +162,25 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
     // eight XCDs), close in time
     const int bid = blockIdx.x;
     const int chunk = bid >> (nz == 2 ? 4 : 3), within = bid - chunk * 8 * nz;   // nz is 1 or 2
-    const int panel = chunk * 8 + (within & 7), z = within >> 3;
-    if (panel >= n_panels) return;
+    const int unit = chunk * 8 + (within & 7), z = within >> 3;
+    if (unit >= n_units) return;
     const int t0 = z * kTok;                       // first token of this workgroup
-    const int nks = gridDim.y, ks = blockIdx.y;
-    // slices of ng / nks groups, the first ng % nks one longer (no division on the device)
-    const int g_begin = ks * slice_base + (ks < slice_extra ? ks : slice_extra);
-    const int g_end = g_begin + slice_base + (ks < slice_extra ? 1 : 0);
+    // Units of work: main_panels panels take their whole K in one workgroup (no atomics); each panel after them is
+    // cut into tail_split slices of K, one workgroup each, which meet in the arrival cells. The launcher picks the
+    // cut so that the workgroups fill whole rounds of the chip. The slices come first in dispatch order: their
+    // critical path has one more trip to memory (the arrival atomics), and trips are short while the chip is still
+    // filling up.
+    const int tail_units = n_units - main_panels;
+    int panel = unit - tail_units, ks = 0, nks = 1, g_begin = 0, g_end = ng;
+    if (unit < tail_units) {
+        const int q = unit / tail_split;
+        panel = main_panels + q;
+        ks = unit - q * tail_split;
+        nks = tail_split;
+        // slices of ng / nks groups, the first ng % nks one longer
+        g_begin = ks * slice_base + (ks < slice_extra ? ks : slice_extra);
+        g_end = g_begin + slice_base + (ks < slice_extra ? 1 : 0);
+    }
 
     // this lane's byte of the panel: half quad >> 1, row l16 (+ 16 per row tile), 8 bytes at (quad & 1) * 8
     const uint8_t *a_base = codes + (size_t) panel * ng * 2048 + (quad >> 1) * 1024 + l16 * 16 + (quad & 1) * 8;
@@ -187,7 +200,16 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
         }
     }
 
-    // the first loads go out before anything that waits (the flag word, the LDS clear)
+    // What the epilogue needs from memory is asked for first: loads return in order, so by the time the first group
+    // of weights is here these are too, and the tail of the kernel has no trip to memory left but its own stores.
+    const int64_t nrow = (int64_t) panel * kPanelRows + lane;
+    const float sw_row = s_w[nrow];                 // rows past N are stored as zero
+    float u_tok[kTok / kWaves];
+#pragma unroll
+    for (int i = 0; i < kTok / kWaves; ++i) u_tok[i] = u[t0 + wave + i * kWaves];   // u has a slot for every padded token
+    const int32_t has_k = *reinterpret_cast<const volatile int32_t *>(flags) & 1;
+
+    // the first loads go out before anything that waits (the LDS clear)
     const int g_first = g_begin + wave;
     const int n = g_first < g_end ? (g_end - g_first + kWaves - 1) / kWaves : 0;
     const int g_last = n > 0 ? g_first + (n - 1) * kWaves : g_begin;
@@ -198,7 +220,7 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
     for (int i = tid; i < 64 * kStride; i += kThreads) s_tot[i] = 0;
 
     if (n > 0) {
-        if (*reinterpret_cast<const volatile int32_t *>(flags) & 1) {
+        if (has_k) {
             stream_slice<TT, true>(ring, a_base, b_base, k_base, Mp, g_first, n, g_last, hi, lo);
         } else {
             stream_slice<TT, false>(ring, a_base, b_base, k_base, Mp, g_first, n, g_last, hi, lo);
@@ -221,8 +243,9 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
     __syncthreads();
 
     // epilogue: lane = row, a wavefront per token (coalesced rows of y); split-K through the arrival cells
-    const int64_t nrow = (int64_t) panel * kPanelRows + lane;
-    for (int tl = wave; tl < kTok; tl += kWaves) {
+#pragma unroll
+    for (int i = 0; i < kTok / kWaves; ++i) {
+        const int tl = wave + i * kWaves;
         const int t = t0 + tl;
         if (t >= M) break;
         int32_t sum = s_tot[lane * kStride + tl];
@@ -235,7 +258,7 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
             __hip_atomic_store(cell, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             sum = (int32_t) (uint32_t) now;
         }
-        if (nrow < N) y[(int64_t) t * ldy + nrow] = (((float) sum * 16.0f) * u[t]) * s_w[nrow];
+        if (nrow < N) y[(int64_t) t * ldy + nrow] = (((float) sum * 16.0f) * u_tok[i]) * sw_row;
     }
 }
 
@@ -243,29 +266,62 @@ template <int TT>
 hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
     const uint8_t *p = a.prepared;
     const int nz = (a.M + TT * 16 - 1) / (TT * 16);
-    const int nks = skinny_ksplit(a.L, a.M);
-    const int blocks = (a.L.n_panels + 7) / 8 * 8 * nz;
-    hipLaunchKernelGGL((rq_skinny_kernel<TT>), dim3(blocks, nks), dim3(kThreads), 0, stream, p + a.L.off_codes,
+    const SkinnyPlan plan = skinny_plan(a.L, a.M);
+    const int n_units = plan.main_panels + (a.L.n_panels - plan.main_panels) * plan.tail_split;
+    const int blocks = (n_units + 7) / 8 * 8 * nz;
+    hipLaunchKernelGGL((rq_skinny_kernel<TT>), dim3(blocks), dim3(kThreads), 0, stream, p + a.L.off_codes,
                        reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,
                        reinterpret_cast<const int32_t *>(p + a.L.off_flags), reinterpret_cast<const uint4 *>(a.act8),
-                       a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels, nz,
-                       reinterpret_cast<unsigned long long *>(a.tot), a.L.n_panels * kPanelRows, a.L.ng / nks, a.L.ng % nks);
+                       a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, n_units, nz,
+                       reinterpret_cast<unsigned long long *>(a.tot), a.L.n_panels * kPanelRows, plan.main_panels,
+                       plan.tail_split, a.L.ng / plan.tail_split, a.L.ng % plan.tail_split);
     return hipGetLastError();
 }
 
 }  // namespace
 
-// K splits across workgroups: enough workgroups to cover the chip twice, within a budget of L2 atomics (one per
-// output and split), and at least two groups per wavefront
-int skinny_ksplit(const PreparedLayout &L, int M) {
+// How the panels are dealt to workgroups. One workgroup keeps a compute unit's memory pipeline full, and workgroups
+// go to the compute units round robin, so the kernel takes as long as the busiest compute unit: 272 whole panels on
+// 256 compute units cost two rounds (measured: 16.9 us against 10.6 us for 256 panels). So the panels that fill
+// whole rounds run as whole-K workgroups, and the remainder is cut along K into slices small enough to spread over
+// the chip: `tail_split` slices per panel, which meet in 64-bit arrival cells. Device-scope atomics cost about 7 ns
+// per thousand, so the cut is chosen by a small cost model (busiest compute unit + atomics) rather than maximised.
+SkinnyPlan skinny_plan(const PreparedLayout &L, int M) {
     static const int forced = getenv("RQ_SKINNY_KSPLIT") ? atoi(getenv("RQ_SKINNY_KSPLIT")) : 0;
+    constexpr int kCUs = 256;
     const int nz = M <= 16 ? 1 : (M + 31) / 32;
-    int nks = (512 + L.n_panels * nz - 1) / (L.n_panels * nz);
-    const int64_t budget = 400000 / ((int64_t) M * L.n_panels * kPanelRows);
-    if (nks > budget) nks = (int) budget;
-    if (forced > 0) nks = forced;
-    if (nks > L.ng / (2 * kWaves)) nks = L.ng / (2 * kWaves);
-    return nks < 1 ? 1 : nks;
+    SkinnyPlan plan;
+    const int smax = L.ng / kWaves < 1 ? 1 : (L.ng / kWaves > 16 ? 16 : L.ng / kWaves);
+    if (forced > 0) {
+        plan.main_panels = 0;
+        plan.tail_split = forced > smax ? smax : forced;
+        return plan;
+    }
+    const int per_round = kCUs / nz;                       // panels in one round of the chip
+    plan.main_panels = L.n_panels / per_round * per_round;
+    plan.tail_split = 1;
+    const int b = L.n_panels - plan.main_panels;
+    if (b == 0) return plan;
+    static const int forced_tail = getenv("RQ_SKINNY_TAIL") ? atoi(getenv("RQ_SKINNY_TAIL")) : 0;
+    if (forced_tail > 0) {
+        plan.tail_split = forced_tail > smax ? smax : forced_tail;
+        return plan;
+    }
+    // microseconds: a panel's weights at the rate one compute unit sustains, atomics at 7 ns per thousand (mostly
+    // hidden behind the whole panels when there are any)
+    const double t_panel = (double) L.ng * 2048.0 / (M <= 16 ? 19000.0 : 13000.0);
+    const double atomics_weight = plan.main_panels > 0 ? 0.25 : 1.0;
+    double best = 1e30;
+    for (int s = 1; s <= smax; ++s) {
+        const int rounds = (b * nz * s + kCUs - 1) / kCUs;
+        const double cost = rounds * t_panel / s
+                            + (s > 1 ? atomics_weight * 0.007e-3 * (double) b * kPanelRows * M * s : 0.0);
+        if (cost < best - 1e-9) {
+            best = cost;
+            plan.tail_split = s;
+        }
+    }
+    return plan;
 }
 
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream) {
