@@ -45,20 +45,29 @@ struct Frag {
     uint4 b[TT][2];    // activation digits (lo, hi) of the token tiles: this lane's quarter
 };
 
+// Addresses are a uniform base (the panel's codes, the digit planes) plus a 32-bit offset per lane. `live` is uniform
+// over the wavefront. A ring slot past the end of the wavefront's share still issues its loads (the loop stays
+// branch-free, so the wait counts stay exact) but with offset 0 in every lane, a few bytes that all lanes share:
+// memory throughput per compute unit is what bounds this kernel, and a ring that fetched real groups past the end
+// would add up to `depth` groups to every wavefront's share.
 template <int TT>
-__device__ __forceinline__ void load_frag(Frag<TT> &f, const uint8_t *a_base, const uint4 *b_base, int g, int Mp) {
+__device__ __forceinline__ void load_frag(Frag<TT> &f, const uint8_t *a_panel, uint32_t a_lane, const uint8_t *b_planes,
+                                          uint32_t b_lane, int g, int Mp, bool live) {
     // weights are read once (twice with two token blocks, and then from L2 at once): non-temporal, so they do not
     // displace the digit planes, which every workgroup re-reads
     typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    const uint32_t ao = live ? a_lane + (uint32_t) g * 2048u : 0u;
+    const uint32_t bo = live ? b_lane + (uint32_t) g * 128u * (uint32_t) Mp : 0u;
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
-        const v2u v = __builtin_nontemporal_load(reinterpret_cast<const v2u *>(a_base + (size_t) g * 2048 + rt * 256));
+        const v2u v = __builtin_nontemporal_load(reinterpret_cast<const v2u *>(a_panel + ao + rt * 256));
         f.a[rt] = make_uint2(v.x, v.y);
     }
+    const uint32_t plane = 64u * (uint32_t) Mp;   // bytes from the low digits of a group to its high digits
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
-        f.b[tt][0] = b_base[(size_t) g * 8 * Mp + 16 * tt];
-        f.b[tt][1] = b_base[(size_t) g * 8 * Mp + (size_t) 4 * Mp + 16 * tt];
+        f.b[tt][0] = *reinterpret_cast<const uint4 *>(b_planes + bo + 256 * tt);
+        f.b[tt][1] = *reinterpret_cast<const uint4 *>(b_planes + bo + plane + 256 * tt);
     }
 }
 
@@ -106,33 +115,32 @@ __device__ __forceinline__ void mma_frag(const Frag<TT> &f, const uint8_t *k_bas
 // One wavefront's share of the K slice: groups g_first, g_first + kWaves, ... (n of them). Ring slot j % D holds
 // group j; the slot is refilled with group j + D as soon as group j's MFMAs have been issued. The scheduling
 // barriers keep the compiler from sinking those loads to their first use (which would expose the whole memory
-// latency once per group). Past the end the ring refetches the last group, and nothing consumes it.
+// latency once per group). Past the end the ring issues idle loads, and nothing consumes them.
 template <int TT>
-__device__ __forceinline__ void fill_ring(Frag<TT> (&ring)[depth_of(TT)], const uint8_t *a_base, const uint4 *b_base,
-                                          int Mp, int g_first, int g_last) {
+__device__ __forceinline__ void fill_ring(Frag<TT> (&ring)[depth_of(TT)], const uint8_t *a_panel, uint32_t a_lane,
+                                          const uint8_t *b_planes, uint32_t b_lane, int Mp, int g_first, int n) {
 #pragma unroll
     for (int i = 0; i < depth_of(TT); ++i) {
-        const int g = g_first + i * kWaves;
-        load_frag<TT>(ring[i], a_base, b_base, g < g_last ? g : g_last, Mp);
+        load_frag<TT>(ring[i], a_panel, a_lane, b_planes, b_lane, g_first + i * kWaves, Mp, i < n);
     }
 }
 
 template <int TT, bool HASK>
-__device__ __forceinline__ void stream_slice(Frag<TT> (&ring)[depth_of(TT)], const uint8_t *a_base,
-                                             const uint4 *b_base, const uint8_t *k_base, int Mp, int g_first, int n,
-                                             int g_last, v4i (&hi)[4][TT], int32_t (&lo)[4][TT][4]) {
+__device__ __forceinline__ void stream_slice(Frag<TT> (&ring)[depth_of(TT)], const uint8_t *a_panel, uint32_t a_lane,
+                                             const uint8_t *b_planes, uint32_t b_lane, const uint8_t *k_base, int Mp,
+                                             int g_first, int n, v4i (&hi)[4][TT], int32_t (&lo)[4][TT][4]) {
     constexpr int D = depth_of(TT);
     // whole rounds of the ring: branch-free, so the wait counts before each group's MFMAs are exact
     const int rounds = n / D;
     for (int r = 0; r < rounds; ++r) {
 #pragma unroll
         for (int i = 0; i < D; ++i) {
-            const int g = g_first + (r * D + i) * kWaves;
-            const int gn = g + D * kWaves;
+            const int j = r * D + i;
+            const int g = g_first + j * kWaves;
             __builtin_amdgcn_sched_barrier(0);
             mma_frag<TT, HASK>(ring[i], k_base, g, hi, lo);
             __builtin_amdgcn_sched_barrier(0);
-            load_frag<TT>(ring[i], a_base, b_base, gn < g_last ? gn : g_last, Mp);
+            load_frag<TT>(ring[i], a_panel, a_lane, b_planes, b_lane, g + D * kWaves, Mp, j + D < n);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -183,9 +191,11 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
     }
 
     // this lane's byte of the panel: half quad >> 1, row l16 (+ 16 per row tile), 8 bytes at (quad & 1) * 8
-    const uint8_t *a_base = codes + (size_t) panel * ng * 2048 + (quad >> 1) * 1024 + l16 * 16 + (quad & 1) * 8;
+    const uint8_t *a_panel = codes + (size_t) panel * ng * 2048;
+    const uint32_t a_lane = (quad >> 1) * 1024 + l16 * 16 + (quad & 1) * 8;
     // this lane's cell of the digit planes: quarter quad, token t0 + l16 (+ 16 per token tile)
-    const uint4 *b_base = act8 + (size_t) quad * Mp + t0 + l16;
+    const uint8_t *b_planes = reinterpret_cast<const uint8_t *>(act8);
+    const uint32_t b_lane = ((uint32_t) quad * Mp + t0 + l16) * 16u;
     const uint8_t *k_base = kmul + (size_t) panel * ng * kPanelRows + 4 * quad;
 
     v4i hi[4][TT];
@@ -212,18 +222,17 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
     // the first loads go out before anything that waits (the LDS clear)
     const int g_first = g_begin + wave;
     const int n = g_first < g_end ? (g_end - g_first + kWaves - 1) / kWaves : 0;
-    const int g_last = n > 0 ? g_first + (n - 1) * kWaves : g_begin;
     Frag<TT> ring[depth_of(TT)];
-    fill_ring<TT>(ring, a_base, b_base, Mp, n > 0 ? g_first : g_begin, g_last);
+    fill_ring<TT>(ring, a_panel, a_lane, b_planes, b_lane, Mp, g_first, n);
     __builtin_amdgcn_sched_barrier(0);
 
     for (int i = tid; i < 64 * kStride; i += kThreads) s_tot[i] = 0;
 
     if (n > 0) {
         if (has_k) {
-            stream_slice<TT, true>(ring, a_base, b_base, k_base, Mp, g_first, n, g_last, hi, lo);
+            stream_slice<TT, true>(ring, a_panel, a_lane, b_planes, b_lane, k_base, Mp, g_first, n, hi, lo);
         } else {
-            stream_slice<TT, false>(ring, a_base, b_base, k_base, Mp, g_first, n, g_last, hi, lo);
+            stream_slice<TT, false>(ring, a_panel, a_lane, b_planes, b_lane, k_base, Mp, g_first, n, hi, lo);
         }
     }
 
@@ -291,7 +300,7 @@ SkinnyPlan skinny_plan(const PreparedLayout &L, int M) {
     constexpr int kCUs = 256;
     const int nz = M <= 16 ? 1 : (M + 31) / 32;
     SkinnyPlan plan;
-    const int smax = L.ng / kWaves < 1 ? 1 : (L.ng / kWaves > 16 ? 16 : L.ng / kWaves);
+    const int smax = L.ng / 4 < 1 ? 1 : (L.ng / 4 > 16 ? 16 : L.ng / 4);   // at least four groups per slice
     if (forced > 0) {
         plan.main_panels = 0;
         plan.tail_split = forced > smax ? smax : forced;
