@@ -141,7 +141,10 @@ class Layer:
         self.x0 = torch.from_numpy(synth.activations("normal", M, 5120, seed)).to(dev)
         self.out = {name: torch.empty((M, N), dtype=torch.float32, device=dev) for name, K, N in self.SHAPES}
         L = rq.load_library()
-        self.ws = torch.empty(max(L.rq_w4a4_workspace_bytes(rq.TYPE_W4A4H, K, N, M) for _, K, N in self.SHAPES),
+        w = self.sets[0]
+        self.ws = torch.empty(max([L.rq_w4a4_workspace_bytes(rq.TYPE_W4A4H, K, N, M) for _, K, N in self.SHAPES] +
+                                  [rq.fused_workspace_bytes([w["q"], w["k"], w["v"]], M),
+                                   rq.fused_workspace_bytes([w["gate"], w["up"]], M)]),
                               dtype=torch.uint8, device=dev)
         self.code_bytes = sum(K * N // 2 for _, K, N in self.SHAPES)
         self.bytes = sum(algorithmic_bytes(K, N, M) for _, K, N in self.SHAPES)

@@ -111,8 +111,10 @@ int rq_w4a4_mul_mat_stages(int type, const void *prepared_dev, int64_t K, int64_
                            void *workspace_dev, size_t workspace_bytes, rq_stream_t stream, int stages);
 
 /* Replaces ggml_cuda_mul_mat_rq_w4a4_fused (P:2371-2380): n <= 3 weights of one type, K, clip and rotation
- * length against the same x (q/k/v, gate/up): one activation transform, then one product per weight.
- * workspace: rq_w4a4_workspace_bytes for the largest N. */
+ * length against the same x (q/k/v, gate/up): one activation transform, then the products.
+ * workspace: rq_w4a4_workspace_bytes for N = the sum of the weights' row counts, each rounded up to 64: the streaming
+ * kernels (M <= 64) then serve all the weights from one launch, as the reference's skinny kernel does. A workspace
+ * sized for the largest N alone is also accepted; the products are then launched one per weight. */
 int rq_w4a4_mul_mat_fused(int type, int n, const void *const *prepared_dev, int64_t K, const int64_t *N,
                           const float *x_dev, int64_t ldx, int64_t M,
                           float *const *y_dev, const int64_t *ldy,

@@ -107,7 +107,21 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     if (!rotation_of(type, K, n_rot, p, m)) return RQ_E_ARGUMENT;
     if (M == 0) return 0;
 
-    const WorkspaceLayout W = workspace_layout(K, Nmax, M);
+    // The streaming kernels serve all the weights of a fused call in one launch when the workspace has split-K cells
+    // for all their rows (rq_w4a4_workspace_bytes with N = the padded sum); with cells for the largest weight only,
+    // the products are launched one after the other. Everything else in the workspace does not depend on N.
+    int64_t Nsum = 0;
+    for (int i = 0; i < n; ++i) Nsum += (N[i] + kPanelRows - 1) / kPanelRows * kPanelRows;
+    WorkspaceLayout W = workspace_layout(K, Nmax, M);
+    bool one_launch = false;
+    if (n > 1) {
+        const WorkspaceLayout Wsum = workspace_layout(K, Nsum, M);
+        if (ws_bytes >= Wsum.bytes) {
+            W = Wsum;
+            one_launch = true;
+        }
+    }
+    const int64_t Ncells = one_launch ? Nsum : Nmax;
     if (ws_bytes < W.bytes || (reinterpret_cast<uintptr_t>(ws) & 255) != 0) return RQ_E_WORKSPACE;
     uint8_t *wsb = reinterpret_cast<uint8_t *>(ws);
 
@@ -155,10 +169,10 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
         q.zero_ptr = reinterpret_cast<int32_t *>(wsb + W.off_tot);
         // only the token slots this call can touch: [min(M, 8)][padded rows] cells of two ints
         const int64_t slots = M < kGemvTokens ? M : kGemvTokens;
-        q.zero_ints = 2 * slots * (int64_t) ((Nmax + kPanelRows - 1) / kPanelRows * kPanelRows);
+        q.zero_ints = 2 * slots * (int64_t) ((Ncells + kPanelRows - 1) / kPanelRows * kPanelRows);
     } else if (path == kPathSkinny) {
         q.zero_ptr = reinterpret_cast<int32_t *>(wsb + W.off_tot);
-        q.zero_ints = 2 * M * (int64_t) ((Nmax + kPanelRows - 1) / kPanelRows * kPanelRows);
+        q.zero_ints = 2 * M * (int64_t) ((Ncells + kPanelRows - 1) / kPanelRows * kPanelRows);
     }
     hipError_t e = hipSuccess;
     if (stages & 1) {
@@ -171,16 +185,24 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     }
     if (!(stages & 2)) return 0;
 
-    for (int i = 0; i < n; ++i) {
-        const PreparedLayout L = prepared_layout(K, N[i]);
+    // launches: one for all weights, or one per weight
+    const int n_launch = one_launch && path != kPathGemm ? 1 : n;
+    for (int l = 0; l < n_launch; ++l) {
+        FusedWeights fw;
+        memset(&fw, 0, sizeof fw);
+        fw.n = n_launch == 1 ? n : 1;
+        for (int j = 0; j < fw.n; ++j) {
+            const int i = n_launch == 1 ? j : l;
+            fw.prepared[j] = reinterpret_cast<const uint8_t *>(prepared[i]);
+            fw.L[j] = prepared_layout(K, N[i]);
+            fw.y[j] = y[i];
+            fw.ldy[j] = ldy[i];
+        }
         if (path == kPathSkinny) {
             SkinnyArgs g;
-            g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
-            g.L = L;
+            g.w = fw;
             g.act8 = wsb + W.off_i8;
             g.u = q.u;
-            g.y = y[i];
-            g.ldy = ldy[i];
             g.M = (int) M;
             g.Mp = act_mp;
             g.tot = reinterpret_cast<int32_t *>(wsb + W.off_tot);
@@ -188,12 +210,12 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             if (e != hipSuccess) return (int) e;
         } else if (gemm) {
             GemmArgs g;
-            g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
-            g.L = L;
+            g.prepared = fw.prepared[0];
+            g.L = fw.L[0];
             g.act8 = wsb + W.off_i8;
             g.u = q.u;
-            g.y = y[i];
-            g.ldy = ldy[i];
+            g.y = fw.y[0];
+            g.ldy = fw.ldy[0];
             g.M = (int) M;
             g.Mp = (int) W.Mp;
             g.groups_per_fold = G / kGroup;
@@ -202,14 +224,12 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
         } else {
             for (int c = 0; c < W.chunks; ++c) {
                 GemvArgs g;
-                g.prepared = reinterpret_cast<const uint8_t *>(prepared[i]);
-                g.L = L;
+                g.w = fw;
+                for (int j = 0; j < fw.n; ++j) g.w.y[j] = fw.y[j] + (int64_t) c * kGemvTokens * fw.ldy[j];
                 g.x = gemv_x + (int64_t) c * kGemvTokens * gemv_ldx;
                 g.ldx = gemv_ldx;
-                g.lohi = q.lohi + (size_t) c * kGemvTokens * L.ng * 2;
+                g.lohi = q.lohi + (size_t) c * kGemvTokens * fw.L[0].ng * 2;
                 g.rpart = q.rpart + (size_t) c * kGemvTokens * kRangeParts;
-                g.y = y[i] + (int64_t) c * kGemvTokens * ldy[i];
-                g.ldy = ldy[i];
                 g.T = (int) (M - (int64_t) c * kGemvTokens < kGemvTokens ? M - (int64_t) c * kGemvTokens : kGemvTokens);
                 g.tot = reinterpret_cast<int32_t *>(wsb + W.off_tot);
                 e = launch_gemv(g, stream);

@@ -151,20 +151,61 @@ hipError_t init_rotate_slab_kernels();
 // digit planes (kActI8 form) from the outputs of launch_rotate_stats: rows in out_f32, ranges in lohi / rpart
 hipError_t launch_quantize_digits(const RotQuantArgs &a, hipStream_t stream);
 
+// Up to three weights of one K served by one launch of a streaming product kernel (q / k / v, gate / up: reference
+// lines 2371-2380). The launch sees one list of panels; panel p belongs to weight w with first[w] <= p < first[w + 1].
+constexpr int kMaxFused = 3;
+struct WeightSet {
+    const uint8_t *codes[kMaxFused];
+    const float   *s_w[kMaxFused];
+    const uint8_t *kmul[kMaxFused];
+    const int32_t *flags[kMaxFused];
+    float         *y[kMaxFused];
+    int64_t        ldy[kMaxFused];
+    int64_t        N[kMaxFused];
+    int            first[kMaxFused + 1];   // unused slots hold the total, so no panel selects them
+    int            ng;
+};
+
+struct FusedWeights {
+    int             n;
+    const uint8_t  *prepared[kMaxFused];
+    PreparedLayout  L[kMaxFused];
+    float          *y[kMaxFused];
+    int64_t         ldy[kMaxFused];
+};
+
+inline WeightSet make_weight_set(const FusedWeights &f) {
+    WeightSet w;
+    int first = 0;
+    for (int i = 0; i < kMaxFused; ++i) {
+        const int k = i < f.n ? i : f.n - 1;   // unused slots repeat the last weight (never selected)
+        const uint8_t *p = f.prepared[k];
+        w.codes[i] = p + f.L[k].off_codes;
+        w.s_w[i] = reinterpret_cast<const float *>(p + f.L[k].off_sw);
+        w.kmul[i] = p + f.L[k].off_kmul;
+        w.flags[i] = reinterpret_cast<const int32_t *>(p + f.L[k].off_flags);
+        w.y[i] = f.y[k];
+        w.ldy[i] = f.ldy[k];
+        w.N[i] = f.L[k].N;
+        w.first[i] = first;
+        if (i < f.n) first += f.L[i].n_panels;
+    }
+    w.first[kMaxFused] = first;
+    w.ng = f.L[0].ng;
+    return w;
+}
+
 struct GemvArgs {
-    const uint8_t  *prepared;
-    PreparedLayout  L;
+    FusedWeights    w;      // y: first token row of this chunk
     const float    *x;      // (rotated) activations of this chunk's first token
     int64_t         ldx;    // row stride in floats
     const float    *lohi;   // clipped group ranges of this chunk's first token, [T][ng][2]
     const float    *rpart;  // partial range maxima of this chunk's first token, [T][kRangeParts]
-    float          *y;      // first token row of this chunk
-    int64_t         ldy;
     int             T;      // 1..8 tokens
     int32_t        *tot;    // split-K cells (zero on entry, left zero)
 };
 hipError_t launch_gemv(const GemvArgs &a, hipStream_t stream);
-int gemv_ksplit(const PreparedLayout &L);
+int gemv_ksplit(int n_panels, int ng);
 
 struct GemmArgs {
     const uint8_t  *prepared;
@@ -180,21 +221,18 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
 
 // up to 64 tokens: MFMA arithmetic on a GEMV-shaped weight stream; same operands as the GEMM plus the split-K cells
 struct SkinnyArgs {
-    const uint8_t  *prepared;
-    PreparedLayout  L;
+    FusedWeights    w;
     const uint8_t  *act8;   // [g][digit][quarter][Mp][16]
     const float    *u;      // [Mp]
-    float          *y;
-    int64_t         ldy;
     int             M, Mp;
-    int32_t        *tot;    // split-K cells [M][n_panels * 64], 64 bits each
+    int32_t        *tot;    // split-K cells [M][panels of all weights * 64], 64 bits each
 };
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream);
 struct SkinnyPlan {
     int main_panels;   // leading panels that run as one whole-K workgroup each
     int tail_split;    // K slices (workgroups) per remaining panel
 };
-SkinnyPlan skinny_plan(const PreparedLayout &L, int M);
+SkinnyPlan skinny_plan(int n_panels, int ng, int M);
 
 hipError_t launch_prepare(const void *blocks, const PreparedLayout &L, uint8_t *prepared, hipStream_t stream);
 

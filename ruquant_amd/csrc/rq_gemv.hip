@@ -98,10 +98,9 @@ __device__ __forceinline__ void compute_batch(const Batch &b, const uint8_t *kp,
 
 template <int T, int kWaves>
 __global__ void __launch_bounds__(kWaves * 64)
-rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
-               const int32_t *__restrict__ flags, const float *__restrict__ x, int64_t ldx,
-               const float *__restrict__ lohi, const float *__restrict__ rpart, float *__restrict__ y, int64_t ldy, int64_t N, int ng,
-               unsigned long long *__restrict__ cells, int n_rows_pad, int slice_base, int slice_extra) {
+rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, const float *__restrict__ lohi,
+               const float *__restrict__ rpart, unsigned long long *__restrict__ cells, int n_rows_pad, int slice_base,
+               int slice_extra) {
     constexpr int NT = kWaves * 64;
     __shared__ int32_t red[kWaves][T][64];
     __shared__ float s_R[T], s_u[T];
@@ -112,7 +111,13 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int panel = blockIdx.x;
+    const int panel = blockIdx.x;          // of the launch: the panels of up to three weights in a row
+    const int wsel = (panel >= ws.first[1]) + (panel >= ws.first[2]);
+    const int wpanel = panel - (wsel == 0 ? 0 : wsel == 1 ? ws.first[1] : ws.first[2]);
+    const uint4 *__restrict__ codes = reinterpret_cast<const uint4 *>(wsel == 0 ? ws.codes[0] : wsel == 1 ? ws.codes[1] : ws.codes[2]);
+    const uint8_t *__restrict__ kmul = wsel == 0 ? ws.kmul[0] : wsel == 1 ? ws.kmul[1] : ws.kmul[2];
+    const int32_t *__restrict__ flags = wsel == 0 ? ws.flags[0] : wsel == 1 ? ws.flags[1] : ws.flags[2];
+    const int ng = ws.ng;
     const int nks = gridDim.y, ks = blockIdx.y;
     // slices of ng / nks groups, the first ng % nks one longer (no division on the device)
     const int g_begin = ks * slice_base + (ks < slice_extra ? ks : slice_extra);
@@ -138,8 +143,8 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
 
     // ... and right behind them the weights of the first batch. This order matters: a wavefront's loads complete in
     // issue order, so the small prologue inputs must be the OLDER loads or they would wait for 10 KiB of weights.
-    const uint4 *wp = codes + (size_t) panel * ng * 128 + lane;
-    const uint8_t *kp = kmul + (size_t) panel * ng * kPanelRows + lane;
+    const uint4 *wp = codes + (size_t) wpanel * ng * 128 + lane;
+    const uint8_t *kp = kmul + (size_t) wpanel * ng * kPanelRows + lane;
     Batch b0;
     load_batch<kWaves>(b0, wp, g_begin + wave, g_end);
 
@@ -210,9 +215,14 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     for (int t = 0; t < T; ++t) red[wave][t][lane] = tot[t];
     __syncthreads();
 
+    const float *__restrict__ s_w = wsel == 0 ? ws.s_w[0] : wsel == 1 ? ws.s_w[1] : ws.s_w[2];
+    float *__restrict__ y = wsel == 0 ? ws.y[0] : wsel == 1 ? ws.y[1] : ws.y[2];
+    const int64_t ldy = wsel == 0 ? ws.ldy[0] : wsel == 1 ? ws.ldy[1] : ws.ldy[2];
+    const int64_t N = wsel == 0 ? ws.N[0] : wsel == 1 ? ws.N[1] : ws.N[2];
     for (int item = tid; item < T * 64; item += NT) {
         const int t = item >> 6;
-        const int64_t n = (int64_t) panel * kPanelRows + lane;
+        const int64_t n = (int64_t) wpanel * kPanelRows + lane;       // row of its weight
+        const int64_t cell_row = (int64_t) panel * kPanelRows + lane;   // row of the launch (split-K cell)
         int32_t sum = 0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) sum += red[w][t][lane];
@@ -222,7 +232,7 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
             // value it returns tells the lane whether it was the last of the nks contributors; that lane alone
             // finishes the output and clears the cell for the next call. No fences, no second round trip: the
             // only cross-workgroup traffic is this one read-modify-write, performed in one place for the chip.
-            unsigned long long *cell = cells + (size_t) t * n_rows_pad + n;
+            unsigned long long *cell = cells + (size_t) t * n_rows_pad + cell_row;
             const unsigned long long mine = (1ull << 48) + (unsigned long long) (long long) sum;
             const unsigned long long now =
                 __hip_atomic_fetch_add(cell, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + mine;
@@ -236,13 +246,11 @@ rq_gemv_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
 
 template <int T, int kWaves>
 hipError_t launch_tw(const GemvArgs &a, int nks, hipStream_t stream) {
-    const uint8_t *p = a.prepared;
-    hipLaunchKernelGGL((rq_gemv_kernel<T, kWaves>), dim3(a.L.n_panels, nks), dim3(kWaves * 64), 0, stream,
-                       reinterpret_cast<const uint4 *>(p + a.L.off_codes),
-                       reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,
-                       reinterpret_cast<const int32_t *>(p + a.L.off_flags), a.x, a.ldx, a.lohi, a.rpart, a.y, a.ldy, a.L.N,
-                       a.L.ng, reinterpret_cast<unsigned long long *>(a.tot), a.L.n_panels * kPanelRows, a.L.ng / nks,
-                       a.L.ng % nks);
+    const WeightSet ws = make_weight_set(a.w);
+    const int n_panels = ws.first[kMaxFused];
+    hipLaunchKernelGGL((rq_gemv_kernel<T, kWaves>), dim3(n_panels, nks), dim3(kWaves * 64), 0, stream, ws, a.x, a.ldx,
+                       a.lohi, a.rpart, reinterpret_cast<unsigned long long *>(a.tot), n_panels * kPanelRows,
+                       ws.ng / nks, ws.ng % nks);
     return hipGetLastError();
 }
 
@@ -262,28 +270,30 @@ hipError_t launch_t(const GemvArgs &a, int nks, hipStream_t stream) {
 // it wants many small workgroups: their starts and tails overlap and the last wave of workgroups is short. Aim for
 // about a thousand workgroups, at least a batch (kGemvWaves x kUnroll groups) each when K allows, at least ten groups
 // per workgroup, and never more than kMaxSlice (the slice's codes live in LDS).
-int gemv_ksplit(const PreparedLayout &L) {
+int gemv_ksplit(int n_panels, int ng) {
     static const int forced = getenv("RQ_GEMV_KSPLIT") ? atoi(getenv("RQ_GEMV_KSPLIT")) : 0;
     int nks;
     if (forced > 0) {
         nks = forced;
     } else {
-        const int by_batch = (L.ng + kGemvWaves * kUnroll - 1) / (kGemvWaves * kUnroll);
-        const int by_grid = (1024 + L.n_panels - 1) / L.n_panels;
+        const int by_batch = (ng + kGemvWaves * kUnroll - 1) / (kGemvWaves * kUnroll);
+        const int by_grid = (1024 + n_panels - 1) / n_panels;
         // more splits than ng / 10 cost more in atomics and short workgroups than they gain in parallelism (measured
         // on 16..96 panels)
-        const int cap = L.ng / 10 > by_batch ? L.ng / 10 : by_batch;
+        const int cap = ng / 10 > by_batch ? ng / 10 : by_batch;
         nks = by_batch > by_grid ? by_batch : by_grid;
         if (nks > cap) nks = cap;
     }
-    const int least = (L.ng + kMaxSlice - 1) / kMaxSlice;   // ceil(ng / nks) <= kMaxSlice
+    const int least = (ng + kMaxSlice - 1) / kMaxSlice;   // ceil(ng / nks) <= kMaxSlice
     if (nks < least) nks = least;
-    if (nks > L.ng) nks = L.ng;
+    if (nks > ng) nks = ng;
     return nks < 1 ? 1 : nks;
 }
 
 hipError_t launch_gemv(const GemvArgs &a, hipStream_t stream) {
-    const int nks = gemv_ksplit(a.L);
+    int n_panels = 0;
+    for (int i = 0; i < a.w.n; ++i) n_panels += a.w.L[i].n_panels;
+    const int nks = gemv_ksplit(n_panels, a.w.L[0].ng);
     switch (a.T) {
         case 1: return launch_t<1>(a, nks, stream);
         case 2: return launch_t<2>(a, nks, stream);

@@ -154,9 +154,8 @@ __device__ __forceinline__ void stream_slice(Frag<TT> (&ring)[depth_of(TT)], con
 
 template <int TT>
 __global__ void __launch_bounds__(kThreads, TT == 1 ? 4 : 2)   // wavefronts per SIMD: two workgroups per CU at TT = 1
-rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
-                 const int32_t *__restrict__ flags, const uint4 *__restrict__ act8, const float *__restrict__ u,
-                 float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng, int n_units, int nz,
+rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const float *__restrict__ u, int M, int Mp,
+                 int n_units, int nz,
                  unsigned long long *__restrict__ cells, int n_rows_pad, int main_panels, int tail_split,
                  int slice_base, int slice_extra) {
     constexpr int kTok = TT * 16;
@@ -178,6 +177,7 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
     // cut so that the workgroups fill whole rounds of the chip. The slices come first in dispatch order: their
     // critical path has one more trip to memory (the arrival atomics), and trips are short while the chip is still
     // filling up.
+    const int ng = ws.ng;
     const int tail_units = n_units - main_panels;
     int panel = unit - tail_units, ks = 0, nks = 1, g_begin = 0, g_end = ng;
     if (unit < tail_units) {
@@ -190,13 +190,24 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
         g_end = g_begin + slice_base + (ks < slice_extra ? 1 : 0);
     }
 
+    // `panel` counts through the panels of up to three weights: which weight, and which of its panels
+    const int wsel = (panel >= ws.first[1]) + (panel >= ws.first[2]);
+    const int wpanel = panel - (wsel == 0 ? 0 : wsel == 1 ? ws.first[1] : ws.first[2]);
+    const uint8_t *__restrict__ codes = wsel == 0 ? ws.codes[0] : wsel == 1 ? ws.codes[1] : ws.codes[2];
+    const uint8_t *__restrict__ kmul = wsel == 0 ? ws.kmul[0] : wsel == 1 ? ws.kmul[1] : ws.kmul[2];
+    const int32_t *__restrict__ flags = wsel == 0 ? ws.flags[0] : wsel == 1 ? ws.flags[1] : ws.flags[2];
+    const float *__restrict__ s_w = wsel == 0 ? ws.s_w[0] : wsel == 1 ? ws.s_w[1] : ws.s_w[2];
+    float *__restrict__ y = wsel == 0 ? ws.y[0] : wsel == 1 ? ws.y[1] : ws.y[2];
+    const int64_t ldy = wsel == 0 ? ws.ldy[0] : wsel == 1 ? ws.ldy[1] : ws.ldy[2];
+    const int64_t N = wsel == 0 ? ws.N[0] : wsel == 1 ? ws.N[1] : ws.N[2];
+
     // this lane's byte of the panel: half quad >> 1, row l16 (+ 16 per row tile), 8 bytes at (quad & 1) * 8
-    const uint8_t *a_panel = codes + (size_t) panel * ng * 2048;
+    const uint8_t *a_panel = codes + (size_t) wpanel * ng * 2048;
     const uint32_t a_lane = (quad >> 1) * 1024 + l16 * 16 + (quad & 1) * 8;
     // this lane's cell of the digit planes: quarter quad, token t0 + l16 (+ 16 per token tile)
     const uint8_t *b_planes = reinterpret_cast<const uint8_t *>(act8);
     const uint32_t b_lane = ((uint32_t) quad * Mp + t0 + l16) * 16u;
-    const uint8_t *k_base = kmul + (size_t) panel * ng * kPanelRows + 4 * quad;
+    const uint8_t *k_base = kmul + (size_t) wpanel * ng * kPanelRows + 4 * quad;
 
     v4i hi[4][TT];
     int32_t lo[4][TT][4];
@@ -212,7 +223,8 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
 
     // What the epilogue needs from memory is asked for first: loads return in order, so by the time the first group
     // of weights is here these are too, and the tail of the kernel has no trip to memory left but its own stores.
-    const int64_t nrow = (int64_t) panel * kPanelRows + lane;
+    const int64_t nrow = (int64_t) wpanel * kPanelRows + lane;      // row of its weight
+    const int64_t cell_row = (int64_t) panel * kPanelRows + lane;   // row of the launch (split-K cell)
     const float sw_row = s_w[nrow];                 // rows past N are stored as zero
     float u_tok[kTok / kWaves];
 #pragma unroll
@@ -259,7 +271,7 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
         if (t >= M) break;
         int32_t sum = s_tot[lane * kStride + tl];
         if (nks > 1) {
-            unsigned long long *cell = cells + (size_t) t * n_rows_pad + nrow;
+            unsigned long long *cell = cells + (size_t) t * n_rows_pad + cell_row;
             const unsigned long long mine = (1ull << 48) + (unsigned long long) (long long) sum;
             const unsigned long long now =
                 __hip_atomic_fetch_add(cell, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + mine;
@@ -273,17 +285,16 @@ rq_skinny_kernel(const uint8_t *__restrict__ codes, const float *__restrict__ s_
 
 template <int TT>
 hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
-    const uint8_t *p = a.prepared;
+    const WeightSet ws = make_weight_set(a.w);
+    const int n_panels = ws.first[kMaxFused];
     const int nz = (a.M + TT * 16 - 1) / (TT * 16);
-    const SkinnyPlan plan = skinny_plan(a.L, a.M);
-    const int n_units = plan.main_panels + (a.L.n_panels - plan.main_panels) * plan.tail_split;
+    const SkinnyPlan plan = skinny_plan(n_panels, ws.ng, a.M);
+    const int n_units = plan.main_panels + (n_panels - plan.main_panels) * plan.tail_split;
     const int blocks = (n_units + 7) / 8 * 8 * nz;
-    hipLaunchKernelGGL((rq_skinny_kernel<TT>), dim3(blocks), dim3(kThreads), 0, stream, p + a.L.off_codes,
-                       reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,
-                       reinterpret_cast<const int32_t *>(p + a.L.off_flags), reinterpret_cast<const uint4 *>(a.act8),
-                       a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, n_units, nz,
-                       reinterpret_cast<unsigned long long *>(a.tot), a.L.n_panels * kPanelRows, plan.main_panels,
-                       plan.tail_split, a.L.ng / plan.tail_split, a.L.ng % plan.tail_split);
+    hipLaunchKernelGGL((rq_skinny_kernel<TT>), dim3(blocks), dim3(kThreads), 0, stream, ws,
+                       reinterpret_cast<const uint4 *>(a.act8), a.u, a.M, a.Mp, n_units, nz,
+                       reinterpret_cast<unsigned long long *>(a.tot), n_panels * kPanelRows, plan.main_panels,
+                       plan.tail_split, ws.ng / plan.tail_split, ws.ng % plan.tail_split);
     return hipGetLastError();
 }
 
@@ -295,21 +306,21 @@ hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
 // whole rounds run as whole-K workgroups, and the remainder is cut along K into slices small enough to spread over
 // the chip: `tail_split` slices per panel, which meet in 64-bit arrival cells. Device-scope atomics cost about 7 ns
 // per thousand, so the cut is chosen by a small cost model (busiest compute unit + atomics) rather than maximised.
-SkinnyPlan skinny_plan(const PreparedLayout &L, int M) {
+SkinnyPlan skinny_plan(int n_panels, int ng, int M) {
     static const int forced = getenv("RQ_SKINNY_KSPLIT") ? atoi(getenv("RQ_SKINNY_KSPLIT")) : 0;
     constexpr int kCUs = 256;
     const int nz = M <= 16 ? 1 : (M + 31) / 32;
     SkinnyPlan plan;
-    const int smax = L.ng / 4 < 1 ? 1 : (L.ng / 4 > 16 ? 16 : L.ng / 4);   // at least four groups per slice
+    const int smax = ng / 4 < 1 ? 1 : (ng / 4 > 16 ? 16 : ng / 4);   // at least four groups per slice
     if (forced > 0) {
         plan.main_panels = 0;
         plan.tail_split = forced > smax ? smax : forced;
         return plan;
     }
     const int per_round = kCUs / nz;                       // panels in one round of the chip
-    plan.main_panels = L.n_panels / per_round * per_round;
+    plan.main_panels = n_panels / per_round * per_round;
     plan.tail_split = 1;
-    const int b = L.n_panels - plan.main_panels;
+    const int b = n_panels - plan.main_panels;
     if (b == 0) return plan;
     static const int forced_tail = getenv("RQ_SKINNY_TAIL") ? atoi(getenv("RQ_SKINNY_TAIL")) : 0;
     if (forced_tail > 0) {
@@ -318,7 +329,7 @@ SkinnyPlan skinny_plan(const PreparedLayout &L, int M) {
     }
     // microseconds: a panel's weights at the rate one compute unit sustains, atomics at 7 ns per thousand (mostly
     // hidden behind the whole panels when there are any)
-    const double t_panel = (double) L.ng * 2048.0 / (M <= 16 ? 19000.0 : 13000.0);
+    const double t_panel = (double) ng * 2048.0 / (M <= 16 ? 19000.0 : 13000.0);
     const double atomics_weight = plan.main_panels > 0 ? 0.25 : 1.0;
     double best = 1e30;
     for (int s = 1; s <= smax; ++s) {

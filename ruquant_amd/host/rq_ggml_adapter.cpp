@@ -105,7 +105,13 @@ void ggml_cuda_mul_mat_rq_w4a4_fused(rq_backend_context &ctx, const rq_tensor *c
         if (Ns[i] > Nmax) Nmax = Ns[i];
     }
     const int64_t K = src0s[0]->ne[0], M = src1->ne[1];
-    const size_t ws_bytes = rq_w4a4_workspace_bytes(src0s[0]->type, K, Nmax, M);
+    // split-K cells for the rows of all weights (each padded to 64): the streaming kernels then take one launch
+    int64_t Nws = Nmax;
+    if (n > 1) {
+        Nws = 0;
+        for (int i = 0; i < n; ++i) Nws += (Ns[i] + 63) / 64 * 64;
+    }
+    const size_t ws_bytes = rq_w4a4_workspace_bytes(src0s[0]->type, K, Nws, M);
     void *ws = scratch(ctx, ws_bytes);
     const int rc = rq_w4a4_mul_mat_fused(src0s[0]->type, n, prepared, K, Ns, (const float *) src1->data,
                                          (int64_t) (src1->nb[1] / sizeof(float)), M, ys, ldys, fu0->clip, fu0->n_rot, ws,

@@ -105,6 +105,15 @@ def mul_mat(weight, x, out=None, workspace=None, clip=None):
     return mul_mat_fused([weight], x, outs=None if out is None else [out], workspace=workspace, clip=clip)[0]
 
 
+def fused_workspace_bytes(weights, M):
+    """Workspace for a fused call that serves all its weights from one launch of the streaming kernels: split-K
+    cells for the rows of every weight (each padded to 64). With room for the largest weight only
+    (rq_w4a4_workspace_bytes of the largest N) the call still works, one product launch per weight."""
+    w0 = weights[0]
+    N = w0.N if len(weights) == 1 else sum((w.N + 63) // 64 * 64 for w in weights)
+    return load_library().rq_w4a4_workspace_bytes(w0.type, w0.K, N, M)
+
+
 def mul_mat_fused(weights, x, outs=None, workspace=None, clip=None):
     """Up to three weights of one type, K, clip and rotation length against the same activations."""
     L = load_library()
@@ -118,9 +127,8 @@ def mul_mat_fused(weights, x, outs=None, workspace=None, clip=None):
     if outs is None:
         outs = [torch.empty((M, w.N), dtype=torch.float32, device=x.device) for w in weights]
     n = len(weights)
-    Nmax = max(w.N for w in weights)
     if workspace is None:
-        workspace = _device_bytes(L.rq_w4a4_workspace_bytes(w0.type, K, Nmax, M), x.device)
+        workspace = _device_bytes(fused_workspace_bytes(weights, M), x.device)
     prepared = (ctypes.c_void_p * n)(*[w.prepared.data_ptr() for w in weights])
     ys = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
     Ns = (ctypes.c_int64 * n)(*[w.N for w in weights])

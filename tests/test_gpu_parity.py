@@ -230,6 +230,40 @@ def test_fused_matches_separate(oracle):
         assert bits_equal(o.cpu().numpy(), want), first_mismatch(o.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("one_launch", [True, False], ids=["one_launch", "launch_per_weight"])
+@pytest.mark.parametrize("M", [1, 3, 5, 8, 16, 23, 40, 64, 130])
+def test_fused_launch_forms(oracle, M, one_launch):
+    """Three weights in one call: legacy headers, weight multipliers (so the per-weight flag word matters) and a row
+    count that is not a multiple of the panel; with split-K cells for all rows (one launch of the streaming kernels)
+    and with cells for the largest weight only (a launch per weight)."""
+    K, type_ = 1536, rq.TYPE_W4A4H
+    rng = np.random.default_rng(M)
+    ws, bl = [], []
+    for i, N in enumerate([384, 96, 1024]):
+        if i == 1:
+            codes = rng.integers(-8, 8, size=(N, K), dtype=np.int8)
+            units = np.abs(rng.normal(0.02, 0.005, size=N)).astype(np.float32)
+            mults = rng.integers(1, 16, size=(N, K // 64), dtype=np.uint8)
+            b = rq.pack_groups(codes, units, mults)
+            rq.set_rot_len(b, K)
+            rq.set_clip(b, 0.9)
+        else:
+            b = synth.random_weight_blocks(N, K, 20 + i, type_, clip=0.9)
+        bl.append(b)
+        ws.append(rq.W4A4Weight(b, type_, DEV))
+    x = synth.activations("student_t4", M, K, 7 + M)
+    xd = torch.from_numpy(x).to(DEV)
+    L = rq.load_library()
+    nbytes = rq.fused_workspace_bytes(ws, M) if one_launch else L.rq_w4a4_workspace_bytes(type_, K, 1024, M)
+    work = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    for rep in range(2):                       # the second call meets the cells the first one left
+        outs = rq.mul_mat_fused(ws, xd, workspace=work)
+        torch.cuda.synchronize()
+        for b, w, o in zip(bl, ws, outs):
+            want = oracle.mul_mat(type_, b, x, w.clip, n_rot=K)
+            assert bits_equal(o.cpu().numpy(), want), first_mismatch(o.cpu().numpy(), want)
+
+
 # ---------------------------------------------------------------- the five benchmark configurations
 
 def test_config1_w4a4_k4096_n1024_m1(oracle):
