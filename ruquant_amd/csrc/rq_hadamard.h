@@ -53,12 +53,22 @@ __device__ __forceinline__ void paley_slice(const float (&col)[P], float (&out)[
     }
 }
 
-template <int P, int S = 0>
-__device__ __forceinline__ void paley_pick(int s, const float (&col)[P], float (&out)[4]) {
+// outputs O * s .. O * s + O - 1 of one column, s uniform over the wavefront: the straight-line code of slice s
+template <int P, int O, int S = 0>
+__device__ __forceinline__ void paley_pick(int s, const float (&col)[P], float (&out)[O]) {
     if (s == S) {
-        paley_slice<P, S>(col, out);
-    } else if constexpr (S + 1 < P / 4) {
-        paley_pick<P, S + 1>(s, col, out);
+        constexpr PaleyTable<P> T = make_paley<P>();
+#pragma unroll
+        for (int o = 0; o < O; ++o) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int i = 0; i < P; ++i) {
+                acc = T.neg[i][O * S + o] ? acc - col[i] : acc + col[i];
+            }
+            out[o] = acc;
+        }
+    } else if constexpr (S + 1 < P / O) {
+        paley_pick<P, O, S + 1>(s, col, out);
     }
 }
 

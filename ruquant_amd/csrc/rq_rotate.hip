@@ -92,7 +92,7 @@ __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs 
 #pragma unroll
             for (int i = 0; i < P; ++i) col[i] = src[i * pm];
             float res[4];
-            paley_pick<P>(s, col, res);
+            paley_pick<P, 4>(s, col, res);
 #pragma unroll
             for (int o = 0; o < 4; ++o) {
                 const int idx = b0 + (4 * s + o) * m;

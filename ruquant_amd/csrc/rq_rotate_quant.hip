@@ -78,10 +78,13 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
             const bool m16 = (m & 15) == 0;
             const int pm = m + (m >> 4);
             if constexpr (SLICED) {
-                // wave-items = (slice of four outputs, run of 64 columns); each wavefront takes a contiguous block
-                // of them, so it stays in one slice's straight-line code for several items in a row
+                // wave-items = (slice of kOut outputs, run of 64 columns); each wavefront takes a contiguous block
+                // of them, so it stays in one slice's straight-line code for several items in a row. Short stages are
+                // cut into four slices: with 256 or 512 columns that is one or two items for each of the sixteen
+                // wavefronts, where slices of four outputs would leave a quarter of them a second item to do alone.
+                constexpr int kOut = P < 44 ? P / 4 : 4;
                 const int col_runs = (ncols + 63) >> 6;
-                const int n_items = (P / 4) * col_runs;
+                const int n_items = (P / kOut) * col_runs;
                 const int per_wave = (n_items + kNT / 64 - 1) / (kNT / 64);
                 const int wave = tid >> 6, lane = tid & 63;
                 for (int it = 0; it < per_wave; ++it) {
@@ -100,10 +103,10 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
 #pragma unroll
                         for (int i = 0; i < P; ++i) col[i] = buf[padi(b0 + i * m)];
                     }
-                    float out[4];
-                    paley_pick<P>(s, col, out);
+                    float out[kOut];
+                    paley_pick<P, kOut>(s, col, out);
 #pragma unroll
-                    for (int o = 0; o < 4; ++o) alt[padi(b0 + (4 * s + o) * m)] = out[o] * a.scale;
+                    for (int o = 0; o < kOut; ++o) alt[padi(b0 + (kOut * s + o) * m)] = out[o] * a.scale;
                 }
                 __syncthreads();
                 float *tmp = buf; buf = alt; alt = tmp;
