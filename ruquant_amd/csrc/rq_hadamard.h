@@ -172,9 +172,36 @@ __device__ __forceinline__ void load_row(float *buf, const float *__restrict__ x
     }
 }
 
-// all Sylvester stages of every chunk of m = 1 << lm floats of a padded row, four stages per trip through LDS
-__device__ __forceinline__ void fwht_row(float *buf, int K, int lm, int tid, int nt) {
-    for (int ls = 0; ls < lm;) {
+// The row from global memory through the first four Sylvester stages (strides 1, 2, 4, 8; chunks of at least 16
+// floats) into the padded LDS row: a thread takes 16 consecutive floats, so the stages run in registers on the way in
+// and the row makes one trip through LDS less. For small batches, where one token's latency is what counts.
+template <int NT>
+__device__ __forceinline__ void load_row_fwht16(float *buf, const float *__restrict__ xr, int K, int tid) {
+    for (int u = tid; u < (K >> 4); u += NT) {
+        const float4 *src = reinterpret_cast<const float4 *>(xr + 16 * u);
+        const float4 q0 = src[0], q1 = src[1], q2 = src[2], q3 = src[3];
+        float v[16] = { q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w, q2.x, q2.y, q2.z, q2.w, q3.x, q3.y, q3.z, q3.w };
+#pragma unroll
+        for (int h = 1; h < 16; h <<= 1) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                if ((j & h) == 0) {
+                    const float lo = v[j], up = v[j + h];
+                    v[j] = lo + up;
+                    v[j + h] = lo - up;
+                }
+            }
+        }
+        float *d = buf + padi(16 * u);   // a run of 16 is contiguous in the padded row
+#pragma unroll
+        for (int j = 0; j < 16; ++j) d[j] = v[j];
+    }
+}
+
+// all Sylvester stages from stride 1 << ls0 up of every chunk of m = 1 << lm floats of a padded row, four stages per
+// trip through LDS
+__device__ __forceinline__ void fwht_row(float *buf, int K, int lm, int tid, int nt, int ls0 = 0) {
+    for (int ls = ls0; ls < lm;) {
         const int lr = lm - ls < 4 ? lm - ls : 4;
         if (lr == 4) fwht_pass<4>(buf, K, lm, ls, tid, nt);
         else if (lr == 3) fwht_pass<3>(buf, K, lm, ls, tid, nt);

@@ -65,13 +65,19 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
     float *g_hi = g_lo + ng;
 
     const float *xr = a.x + (int64_t) t * a.ldx;
-    load_row<kNT>(buf, xr, K, tid);
+    // small batches: the first four Sylvester stages ride on the load (one trip through LDS less per token)
+    const bool fused_first = SLICED && a.rotate && (a.m & 15) == 0;
+    if (fused_first) {
+        load_row_fwht16<kNT>(buf, xr, K, tid);
+    } else {
+        load_row<kNT>(buf, xr, K, tid);
+    }
     __syncthreads();
 
     if (a.rotate) {
         const int m = a.m;
         const int lm = __ffs(m) - 1;
-        fwht_row(buf, K, lm, tid, kNT);
+        fwht_row(buf, K, lm, tid, kNT, fused_first ? 4 : 0);
         if constexpr (P > 1) {
             // Paley across the P chunks of every rotation block (reference lines 2466-2482), then the scale
             const int ncols = K / P;  // columns of all rotation blocks of this token
