@@ -57,9 +57,10 @@ __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs 
     const int wave = tid >> 6, lane = tid & 63;
 
     const float *xr = a.x + (int64_t) t * a.ldx;
-    load_row<kRT>(buf, xr, K, tid);
+    // the first four Sylvester stages ride on the load (chunks here are multiples of 64)
+    load_row_fwht16<kRT>(buf, xr, K, tid);
     __syncthreads();
-    fwht_row(buf, K, lm, tid, kRT);
+    fwht_row(buf, K, lm, tid, kRT, 4);
 
     float *out = a.out_f32 + (int64_t) t * a.ldo;
     float *lh = a.lohi + (size_t) t * ng * 2;
