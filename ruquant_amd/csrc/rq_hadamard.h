@@ -95,11 +95,30 @@ __device__ __forceinline__ void paley_column_generic(const float (&col)[P], floa
     if constexpr (S + 1 < P / 4) paley_column_generic<P, S + 1, TR>(col, buf, b0, m, scale);
 }
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
+// Wavefront-wide max / min, the same value in every lane. The steps are DPP lane permutations (swap within pairs,
+// within quads, mirror the half rows, mirror the rows of 16, then carry across rows), which run at vector-ALU speed;
+// six dependent LDS-crossbar permutes would cost several hundred cycles each time, and the rotation kernels reduce
+// once per activation group.
+template <bool MAX>
+__device__ __forceinline__ float wave_reduce(float v) {
+#define RQ_DPP_STEP(ctrl, row_mask)                                                                              \
+    {                                                                                                            \
+        const float o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v),         \
+                                                                              __builtin_bit_cast(int, v), ctrl,  \
+                                                                              row_mask, 0xF, false));            \
+        v = MAX ? fmaxf(v, o) : fminf(v, o);                                                                     \
+    }
+    RQ_DPP_STEP(0xB1, 0xF)    // quad_perm [1, 0, 3, 2]
+    RQ_DPP_STEP(0x4E, 0xF)    // quad_perm [2, 3, 0, 1]
+    RQ_DPP_STEP(0x141, 0xF)   // row_half_mirror
+    RQ_DPP_STEP(0x140, 0xF)   // row_mirror: every lane of a row now holds the row's value
+    RQ_DPP_STEP(0x142, 0xA)   // row_bcast:15 into rows 1 and 3
+    RQ_DPP_STEP(0x143, 0xC)   // row_bcast:31 into rows 2 and 3: lane 63 holds the wavefront's value
+#undef RQ_DPP_STEP
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+__device__ __forceinline__ float wave_max(float v) { return wave_reduce<true>(v); }
+__device__ __forceinline__ float wave_min(float v) { return wave_reduce<false>(v); }
 
 // The row sits in LDS with one float of padding after every 16: element i lives at i + i / 16. With it the
 // strided accesses of the register butterflies (16 elements 16, 256, ... apart) spread over all banks.

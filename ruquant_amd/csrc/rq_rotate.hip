@@ -19,17 +19,6 @@ using namespace had;
 
 constexpr int kRT = 512;  // threads per workgroup
 
-__device__ __forceinline__ float wave_min(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fminf(v, __shfl_xor(v, off, 64));
-    return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
-}
-
 template <int P>
 __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs a, int slabs, int parts) {
     extern __shared__ __align__(16) float buf[];
