@@ -232,7 +232,7 @@ struct SkinnyPlan {
     int main_panels;   // leading panels that run as one whole-K workgroup each
     int tail_split;    // K slices (workgroups) per remaining panel
 };
-SkinnyPlan skinny_plan(int n_panels, int ng, int M);
+SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz);
 
 hipError_t launch_prepare(const void *blocks, const PreparedLayout &L, uint8_t *prepared, hipStream_t stream);
 

@@ -288,7 +288,7 @@ hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
     const WeightSet ws = make_weight_set(a.w);
     const int n_panels = ws.first[kMaxFused];
     const int nz = (a.M + TT * 16 - 1) / (TT * 16);
-    const SkinnyPlan plan = skinny_plan(n_panels, ws.ng, a.M);
+    const SkinnyPlan plan = skinny_plan(n_panels, ws.ng, a.M, nz);
     const int n_units = plan.main_panels + (n_panels - plan.main_panels) * plan.tail_split;
     const int blocks = (n_units + 7) / 8 * 8 * nz;
     hipLaunchKernelGGL((rq_skinny_kernel<TT>), dim3(blocks), dim3(kThreads), 0, stream, ws,
@@ -306,10 +306,9 @@ hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
 // whole rounds run as whole-K workgroups, and the remainder is cut along K into slices small enough to spread over
 // the chip: `tail_split` slices per panel, which meet in 64-bit arrival cells. Device-scope atomics cost about 7 ns
 // per thousand, so the cut is chosen by a small cost model (busiest compute unit + atomics) rather than maximised.
-SkinnyPlan skinny_plan(int n_panels, int ng, int M) {
+SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz) {
     static const int forced = getenv("RQ_SKINNY_KSPLIT") ? atoi(getenv("RQ_SKINNY_KSPLIT")) : 0;
     constexpr int kCUs = 256;
-    const int nz = M <= 16 ? 1 : (M + 31) / 32;
     SkinnyPlan plan;
     const int smax = ng / 4 < 1 ? 1 : (ng / 4 > 16 ? 16 : ng / 4);   // at least four groups per slice
     if (forced > 0) {
@@ -345,7 +344,8 @@ SkinnyPlan skinny_plan(int n_panels, int ng, int M) {
 }
 
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream) {
-    if (a.M <= 16) return launch_tt<1>(a, stream);
+    static const int tt1_max = getenv("RQ_SKINNY_TT1_MAX") ? atoi(getenv("RQ_SKINNY_TT1_MAX")) : 16;
+    if (a.M <= (tt1_max > 32 ? 32 : tt1_max)) return launch_tt<1>(a, stream);
     return launch_tt<2>(a, stream);
 }
 
