@@ -25,9 +25,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
-# HBM bytes per launch of the headline product kernel: rocprofv3 FETCH_SIZE 21,928.6 KiB / 0.500 (scale from a plain
+# HBM bytes per launch of the headline product kernel: rocprofv3 FETCH_SIZE 21,923.0 KiB / 0.500 (scale from a plain
 # copy of known size) + WRITE_SIZE 748.0 KiB / 1.000, from the runs summarized in profiles/gemv_m1_k5120_n17408.md
-HEADLINE_TRAFFIC_BYTES = int((21928.6 / 0.500 + 748.0) * 1024)
+HEADLINE_TRAFFIC_BYTES = int((21923.0 / 0.500 + 748.0) * 1024)
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA
 
 
