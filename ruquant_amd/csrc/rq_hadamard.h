@@ -72,14 +72,23 @@ __device__ __forceinline__ void paley_pick(int s, const float (&col)[P], float (
     }
 }
 
-// all P outputs of one column, written back in place (the column is private to the calling thread)
-template <int P, int S = 0, bool TR = false>
+// all P outputs of one column, written back in place (the column is private to the calling thread). STRIDE is the
+// distance between the chunks of a column in the padded row when it is known at compile time (0: use `stride`): the
+// P loads and P stores then share one or two address registers with immediate offsets, where a run-time stride costs
+// an address register per element, which for long columns is what spills.
+template <int P, int S = 0, bool TR = false, int STRIDE = 0>
 __device__ __forceinline__ void paley_column(const float (&col)[P], float *dst, int stride, float scale) {
     float out[4];
     paley_slice<P, S, TR>(col, out);
 #pragma unroll
-    for (int o = 0; o < 4; ++o) dst[(4 * S + o) * stride] = out[o] * scale;
-    if constexpr (S + 1 < P / 4) paley_column<P, S + 1, TR>(col, dst, stride, scale);
+    for (int o = 0; o < 4; ++o) dst[(4 * S + o) * (STRIDE ? STRIDE : stride)] = out[o] * scale;
+    if constexpr (S + 1 < P / 4) paley_column<P, S + 1, TR, STRIDE>(col, dst, stride, scale);
+}
+
+template <int P, int STRIDE>
+__device__ __forceinline__ void load_column(float (&col)[P], const float *src, int stride) {
+#pragma unroll
+    for (int i = 0; i < P; ++i) col[i] = src[i * (STRIDE ? STRIDE : stride)];
 }
 
 // same, for chunk lengths that are not a multiple of 16 (the padded stride is then not uniform)

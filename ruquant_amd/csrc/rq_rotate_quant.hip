@@ -121,10 +121,13 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
                     const int rb = cidx / m, j = cidx - rb * m;
                     const int b0 = rb * a.n_rot + j;
                     float col[P];
-                    if (m16) {
+                    if (pm == 272) {   // chunks of 256 (K = 5120, 17408): the common case, compile-time stride
                         float *src = buf + padi(b0);
-#pragma unroll
-                        for (int i = 0; i < P; ++i) col[i] = src[i * pm];
+                        load_column<P, 272>(col, src, pm);
+                        paley_column<P, 0, false, 272>(col, src, pm, a.scale);
+                    } else if (m16) {
+                        float *src = buf + padi(b0);
+                        load_column<P, 0>(col, src, pm);
                         paley_column<P>(col, src, pm, a.scale);
                     } else {
 #pragma unroll
