@@ -65,8 +65,8 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
     float *g_hi = g_lo + ng;
 
     const float *xr = a.x + (int64_t) t * a.ldx;
-    // small batches: the first four Sylvester stages ride on the load (one trip through LDS less per token)
-    const bool fused_first = SLICED && a.rotate && (a.m & 15) == 0;
+    // the first four Sylvester stages ride on the load (one trip through LDS less per token)
+    const bool fused_first = a.rotate && (a.m & 15) == 0;
     if (fused_first) {
         load_row_fwht16<kNT>(buf, xr, K, tid);
     } else {
