@@ -164,6 +164,33 @@ __device__ __forceinline__ void fwht_pass(float *buf, int K, int lm, int ls, int
 }
 
 
+// Eight consecutive values of one activation group -> the two int8 digit words pairs of the MFMA operand layout.
+// q = clamp(rint(x * inv) + zf, 0, 15) as the reference computes it (patch lines 2670-2675); p = m (q - z), |p| <= 3825,
+// is formed in fp32 (small integers: exact) and split into balanced digits p = 64 hi + lo, lo in [-32, 31]. Bytes go
+// in the order the weight unpack yields: the even values of the word (`*_e`), then the odd ones (`*_o`); v_perm_b32
+// gathers four low bytes in three instructions.
+__device__ __forceinline__ uint32_t pack_low_bytes(int x0, int x1, int x2, int x3) {
+    const uint32_t t0 = __builtin_amdgcn_perm((uint32_t) x1, (uint32_t) x0, 0x0c0c0400u);
+    const uint32_t t1 = __builtin_amdgcn_perm((uint32_t) x3, (uint32_t) x2, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(t1, t0, 0x05040100u);
+}
+
+__device__ __forceinline__ void digits_of_word(const float (&f)[8], float inv, float zf, float mgf, uint32_t &lo_e,
+                                               uint32_t &lo_o, uint32_t &hi_e, uint32_t &hi_o) {
+    int lo[8], hi[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float q = fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
+        const int p = (int) ((q - zf) * mgf);
+        hi[j] = (p + 32) >> 6;
+        lo[j] = p - (hi[j] << 6);
+    }
+    lo_e = pack_low_bytes(lo[0], lo[2], lo[4], lo[6]);
+    lo_o = pack_low_bytes(lo[1], lo[3], lo[5], lo[7]);
+    hi_e = pack_low_bytes(hi[0], hi[2], hi[4], hi[6]);
+    hi_o = pack_low_bytes(hi[1], hi[3], hi[5], hi[7]);
+}
+
 // Workgroup barrier for data that travels through LDS only: waits for this wavefront's LDS operations, not for its
 // outstanding global loads (which __syncthreads() would also drain, stalling a kernel that keeps weight loads in
 // flight across its prologue).

@@ -128,28 +128,11 @@ __global__ void __launch_bounds__(kRT) rq_quantize_digits_kernel(const RotQuantA
     const int mg = (int) fminf(fmaxf(ceilf(((lh.y - lh.x) * 255.0f) / R), 1.0f), 255.0f);
     const float inv = 1.0f / ((float) mg * u);
     const float zf = fminf(fmaxf(rintf(-lh.x * inv), 0.0f), 15.0f);
-    const int z = (int) zf;
     const float4 *src = reinterpret_cast<const float4 *>(a.out_f32 + (int64_t) t * a.ldo + 8 * w);
     const float4 v0 = src[0], v1 = src[1];
     const float f[8] = { v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w };
-    uint32_t lo_e = 0, lo_o = 0, hi_e = 0, hi_o = 0;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int q = (int) fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
-        // p = m (q - z), |p| <= 3825, as two balanced int8 digits p = 64 hi + lo, lo in [-32, 31]; bytes in the
-        // order the weight unpack yields: the even codes of the word, then the odd codes
-        const int p = mg * (q - z);
-        const int lo = ((p + 32) & 63) - 32;
-        const int hi = (p - lo) >> 6;
-        const int sh = 8 * (j >> 1);
-        if (j & 1) {
-            lo_o |= (uint32_t) (lo & 0xFF) << sh;
-            hi_o |= (uint32_t) (hi & 0xFF) << sh;
-        } else {
-            lo_e |= (uint32_t) (lo & 0xFF) << sh;
-            hi_e |= (uint32_t) (hi & 0xFF) << sh;
-        }
-    }
+    uint32_t lo_e, lo_o, hi_e, hi_o;
+    digits_of_word(f, inv, zf, (float) mg, lo_e, lo_o, hi_e, hi_o);
     // [group][digit][quarter of the group][token][16 bytes]
     const size_t cell = (((size_t) g * 2 + 0) * 4 + ((w & 7) >> 1)) * a.Mp + t;
     uint32_t *dst = a.act + cell * 4 + (w & 1) * 2;

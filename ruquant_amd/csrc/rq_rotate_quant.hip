@@ -222,28 +222,9 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
         const int z = (int) zf;
         const float *sp = buf + padi(8 * wc);
         const float f[8] = { sp[0], sp[1], sp[2], sp[3], sp[4], sp[5], sp[6], sp[7] };
-        int q[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) q[j] = (int) fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
-
         if (a.mode == kActI8) {
-            // p = m (q - z), |p| <= 3825, as two balanced int8 digits p = 64 hi + lo, lo in [-32, 31]; bytes in the
-            // order the weight unpack yields: the even codes of the word, then the odd codes
-            uint32_t lo_e = 0, lo_o = 0, hi_e = 0, hi_o = 0;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int p = mg * (q[j] - z);
-                const int lo = ((p + 32) & 63) - 32;
-                const int hi = (p - lo) >> 6;
-                const int sh = 8 * (j >> 1);
-                if (j & 1) {
-                    lo_o |= (uint32_t) (lo & 0xFF) << sh;
-                    hi_o |= (uint32_t) (hi & 0xFF) << sh;
-                } else {
-                    lo_e |= (uint32_t) (lo & 0xFF) << sh;
-                    hi_e |= (uint32_t) (hi & 0xFF) << sh;
-                }
-            }
+            uint32_t lo_e, lo_o, hi_e, hi_o;
+            digits_of_word(f, inv, zf, (float) mg, lo_e, lo_o, hi_e, hi_o);
             if (on) {
                 // [group][digit][quarter of the group][token][16 bytes]: a token tile of one quarter is contiguous
                 const size_t cell = (((size_t) g * 2 + 0) * 4 + ((w & 7) >> 1)) * a.Mp + t;
@@ -256,7 +237,10 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
 
         uint32_t word = 0;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) word |= (uint32_t) ((q[j] - 8) & 0xF) << (4 * j);
+        for (int j = 0; j < 8; ++j) {
+            const int q = (int) fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
+            word |= (uint32_t) ((q - 8) & 0xF) << (4 * j);
+        }
 
         {  // kActBlocks: the reference's A4 / A4H storage (reference lines 2656-2661, 2667-2669)
             const int base = tid & 32;  // lanes base, base + lpg, ... hold the block's 4, 2 or 1 groups
