@@ -314,9 +314,11 @@ def test_config4_down_projection(oracle, M):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
-def test_config5_transformer_layer_chain(oracle):
-    """Seven matmuls at M = 16 chained along the layer's dataflow: q, k, v <- x0; o <- q; gate, up <- o; down <- up."""
-    M, type_ = 16, rq.TYPE_W4A4H
+@pytest.mark.parametrize("M", [16, 1, 5, 40])
+def test_config5_transformer_layer_chain(oracle, M):
+    """Seven matmuls chained along the layer's dataflow: q, k, v <- x0; o <- q; gate, up <- o; down <- up. M = 16 is the
+    benchmark configuration; 1 and 5 take the GEMV (fused calls in one launch), 40 the two-token-block skinny kernel."""
+    type_ = rq.TYPE_W4A4H
     shapes = dict(q=(5120, 6144), k=(5120, 1024), v=(5120, 1024), o=(6144, 5120), gate=(5120, 17408),
                   up=(5120, 17408), down=(17408, 5120))
     blocks = {n: synth.random_weight_blocks(No, Ki, 100 + i, type_) for i, (n, (Ki, No)) in enumerate(shapes.items())}
