@@ -12,7 +12,7 @@ Prints one JSON line. Besides the contract fields it carries
   cpu_baseline : the CPU oracle (a bit-identical restatement of the ggml-cpu reference path) on the host cores,
   extra        : the same measurements for the other benchmark shapes (M = 2048 prefill as TOPS against the dense
                  int8 MFMA peak, the N = 5120 decode shapes, the K = 17408 down projection) and the seven matmuls of
-                 one transformer layer at 16 tokens, run in the layer's dataflow.
+                 one transformer layer at 16 tokens and at one token, run in the layer's dataflow.
 """
 import argparse
 import json
@@ -300,10 +300,13 @@ def main():
             steps = args.steps if m <= 64 else max(5, args.steps // 10)
             extra[name], _, _ = measure(head, steps, min(args.warmup, steps), bound)
 
-        if not want or "layer_m16" in want:
-            head = None
-            torch.cuda.empty_cache()
-            extra["layer_m16"] = Layer(16).measure(max(5, args.steps // 4), 3)
+        for name, m in (("layer_m16", 16), ("layer_m1", 1)):
+            if not want or name in want:
+                head = None
+                torch.cuda.empty_cache()
+                layer = Layer(m)
+                extra[name] = layer.measure(max(5, args.steps // 4), 3)
+                del layer
 
     line = {
         "metric": "w4a4h_matmul_gbps_m1", "value": round(b / op_ms / 1e6, 1), "unit": "GB/s",
