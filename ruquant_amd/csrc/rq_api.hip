@@ -206,6 +206,8 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             g.M = (int) M;
             g.Mp = act_mp;
             g.tot = reinterpret_cast<int32_t *>(wsb + W.off_tot);
+            g.panel0 = 0;
+            g.panels = 0;
             e = launch_skinny(g, stream);
             if (e != hipSuccess) return (int) e;
         } else if (gemm) {

@@ -226,6 +226,9 @@ struct SkinnyArgs {
     const float    *u;      // [Mp]
     int             M, Mp;
     int32_t        *tot;    // split-K cells [M][panels of all weights * 64], 64 bits each
+    // a sub-range of the (single) weight's panels, whole K per workgroup, any number of 32-token blocks: the tail of
+    // a GEMM launch (rq_gemm.hip). panels == 0: all panels, planned by skinny_plan.
+    int             panel0, panels;
 };
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream);
 struct SkinnyPlan {

@@ -26,6 +26,8 @@
 // contiguous on both sides.
 #include "rq_common.h"
 
+#include <string.h>
+
 #include <stdlib.h>
 
 #pragma clang fp contract(off)
@@ -535,6 +537,22 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     if (cost(n_tiles) < cost(n_wide)) n_wide = n_tiles;
     if (force == 0) n_wide = n_tiles;
     if (force == 1 || a.groups_per_fold > 1) n_wide = 0;   // wider activation groups: narrow tiles only
+    // A third way to run the rows that the whole wide rounds leave over: the skinny kernel (rq_skinny.hip), a
+    // workgroup per panel of 64 rows and block of 32 tokens, whole K, no LDS staging. A round of 256 of those takes
+    // about 0.65 of a narrow round (measured: 20 us against 31 us at K = 5120) but holds an eighth of a narrow tile
+    // each: it wins when the leftover is a few row tiles and the token count moderate (K=5120, N=17408, M=512: 256
+    // wide tiles + 16 panels x 16 token blocks, 116.6 -> 102.4 us; at M=1024 the narrow tiles stay ahead).
+    static const int skinny_tail_on = getenv("RQ_GEMM_SKINNY_TAIL") ? atoi(getenv("RQ_GEMM_SKINNY_TAIL")) : 1;
+    bool skinny_tail = false;
+    if (skinny_tail_on && force < 0 && a.groups_per_fold == 1 && whole > 0 && whole < n_tiles) {
+        const int tail_panels = a.L.n_panels - whole / n_tok_tiles * 4;
+        const int64_t wgs = (int64_t) tail_panels * ((a.M + 31) / 32);
+        const double c = 2.6 * (whole / kCUs) + 0.65 * ((wgs + kCUs - 1) / kCUs);
+        if (c < cost(n_wide)) {
+            n_wide = whole;
+            skinny_tail = true;
+        }
+    }
     // the super-tile order of the wide kernel needs a wide region of whole blocks of 8 row tiles x 4 token tiles
     static const int no_super = getenv("RQ_GEMM_SUPER") ? atoi(getenv("RQ_GEMM_SUPER")) == 0 : 0;
     const int super_tiles = !no_super && n_wide > 0 && n_tok_tiles % 4 == 0 && n_wide % n_tok_tiles == 0 &&
@@ -547,6 +565,23 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
         hipLaunchKernelGGL(rq_gemm_kernel<false>, dim3(n_wide), dim3(kThreads), 0, stream, codes, s_w,
                            p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
                            n_tok_tiles, 0, n_wide, super_tiles, 4);
+    }
+    if (n_wide < n_tiles && skinny_tail) {
+        SkinnyArgs t;
+        memset(&t, 0, sizeof t);
+        t.w.n = 1;
+        t.w.prepared[0] = a.prepared;
+        t.w.L[0] = a.L;
+        t.w.y[0] = a.y;
+        t.w.ldy[0] = a.ldy;
+        t.act8 = a.act8;
+        t.u = a.u;
+        t.M = a.M;
+        t.Mp = a.Mp;
+        t.tot = nullptr;   // whole K per workgroup
+        t.panel0 = n_wide / n_tok_tiles * 4;
+        t.panels = a.L.n_panels - t.panel0;
+        return launch_skinny(t, stream);
     }
     if (n_wide < n_tiles) {
         const int n_blocks = (n_row_tiles - n_wide / n_tok_tiles) * per_row;

@@ -157,7 +157,7 @@ __global__ void __launch_bounds__(kThreads, TT == 1 ? 4 : 2)   // wavefronts per
 rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const float *__restrict__ u, int M, int Mp,
                  int n_units, int nz,
                  unsigned long long *__restrict__ cells, int n_rows_pad, int main_panels, int tail_split,
-                 int slice_base, int slice_extra) {
+                 int slice_base, int slice_extra, int panel0) {
     constexpr int kTok = TT * 16;
     constexpr int kStride = kTok + 1;             // padded: the epilogue reads a column of this array
     __shared__ int32_t s_tot[64 * kStride];
@@ -168,7 +168,8 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const float
     // workgroups of one panel's token blocks sit 8 apart in dispatch order: same XCD (ids go round-robin over the
     // eight XCDs), close in time
     const int bid = blockIdx.x;
-    const int chunk = bid >> (nz == 2 ? 4 : 3), within = bid - chunk * 8 * nz;   // nz is 1 or 2
+    const int chunk = nz == 1 ? bid >> 3 : nz == 2 ? bid >> 4 : bid / (8 * nz);
+    const int within = bid - chunk * 8 * nz;
     const int unit = chunk * 8 + (within & 7), z = within >> 3;
     if (unit >= n_units) return;
     const int t0 = z * kTok;                       // first token of this workgroup
@@ -190,6 +191,7 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const float
         g_end = g_begin + slice_base + (ks < slice_extra ? 1 : 0);
     }
 
+    panel += panel0;   // a launch over a sub-range of the panels (the tail of a GEMM launch)
     // `panel` counts through the panels of up to three weights: which weight, and which of its panels
     const int wsel = (panel >= ws.first[1]) + (panel >= ws.first[2]);
     const int wpanel = panel - (wsel == 0 ? 0 : wsel == 1 ? ws.first[1] : ws.first[2]);
@@ -286,15 +288,22 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const float
 template <int TT>
 hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
     const WeightSet ws = make_weight_set(a.w);
-    const int n_panels = ws.first[kMaxFused];
+    const int n_panels = a.panels > 0 ? a.panels : ws.first[kMaxFused];
     const int nz = (a.M + TT * 16 - 1) / (TT * 16);
-    const SkinnyPlan plan = skinny_plan(n_panels, ws.ng, a.M, nz);
+    SkinnyPlan plan;
+    if (a.panels > 0) {   // whole K per workgroup: no arrival cells
+        plan.main_panels = n_panels;
+        plan.tail_split = 1;
+    } else {
+        plan = skinny_plan(n_panels, ws.ng, a.M, nz);
+    }
     const int n_units = plan.main_panels + (n_panels - plan.main_panels) * plan.tail_split;
     const int blocks = (n_units + 7) / 8 * 8 * nz;
     hipLaunchKernelGGL((rq_skinny_kernel<TT>), dim3(blocks), dim3(kThreads), 0, stream, ws,
                        reinterpret_cast<const uint4 *>(a.act8), a.u, a.M, a.Mp, n_units, nz,
-                       reinterpret_cast<unsigned long long *>(a.tot), n_panels * kPanelRows, plan.main_panels,
-                       plan.tail_split, ws.ng / plan.tail_split, ws.ng % plan.tail_split);
+                       reinterpret_cast<unsigned long long *>(a.tot), ws.first[kMaxFused] * kPanelRows,
+                       plan.main_panels, plan.tail_split, ws.ng / plan.tail_split, ws.ng % plan.tail_split,
+                       a.panels > 0 ? a.panel0 : 0);
     return hipGetLastError();
 }
 
@@ -345,6 +354,7 @@ SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz) {
 
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream) {
     static const int tt1_max = getenv("RQ_SKINNY_TT1_MAX") ? atoi(getenv("RQ_SKINNY_TT1_MAX")) : 16;
+    if (a.panels > 0) return launch_tt<2>(a, stream);   // the tail of a GEMM launch: blocks of 32 tokens
     if (a.M <= (tt1_max > 32 ? 32 : tt1_max)) return launch_tt<1>(a, stream);
     return launch_tt<2>(a, stream);
 }

@@ -341,6 +341,19 @@ def test_config5_transformer_layer_chain(oracle, M):
         assert bits_equal(g, want), name + ": " + first_mismatch(g, want)
 
 
+@pytest.mark.parametrize("wgroup", [0, 64], ids=["legacy", "wgroup64"])
+@pytest.mark.parametrize("N,M", [(8300, 1024), (16500, 520)])
+def test_gemm_leftover_rows(oracle, N, M, wgroup):
+    """More than 256 wide tiles with a few rows left over: whole wide rounds plus a tail that runs through the skinny
+    kernel (a sub-range of the panels, blocks of 32 tokens, the last panel partly filled)."""
+    K, type_ = 256, rq.TYPE_W4A4H
+    blocks, wf, W = _weights(oracle, N, K, type_, wgroup=wgroup)
+    x = adversarial_activations(M, K, type_, wf, seed=N + M)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=K)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
 # ---------------------------------------------------------------- properties that hold at any size
 
 @pytest.mark.parametrize("M", [1, 8, 16, 200])
