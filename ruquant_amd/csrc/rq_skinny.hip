@@ -355,7 +355,7 @@ SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz) {
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream) {
     static const int tt1_max = getenv("RQ_SKINNY_TT1_MAX") ? atoi(getenv("RQ_SKINNY_TT1_MAX")) : 16;
     if (a.panels > 0) return launch_tt<2>(a, stream);   // the tail of a GEMM launch: blocks of 32 tokens
-    if (a.M <= (tt1_max > 32 ? 32 : tt1_max)) return launch_tt<1>(a, stream);
+    if (a.M <= (tt1_max > 64 ? 64 : tt1_max)) return launch_tt<1>(a, stream);
     return launch_tt<2>(a, stream);
 }
 
