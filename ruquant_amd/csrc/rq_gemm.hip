@@ -544,7 +544,9 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     // wide tiles + 16 panels x 16 token blocks, 116.6 -> 102.4 us; at M=1024 the narrow tiles stay ahead).
     static const int skinny_tail_on = getenv("RQ_GEMM_SKINNY_TAIL") ? atoi(getenv("RQ_GEMM_SKINNY_TAIL")) : 1;
     bool skinny_tail = false;
-    if (skinny_tail_on && force < 0 && a.groups_per_fold == 1 && whole > 0 && whole < n_tiles) {
+    // (the skinny kernel addresses the digit planes with 32-bit offsets)
+    const bool planes_fit = (int64_t) a.L.ng * 128 * a.Mp < ((int64_t) 1 << 32);
+    if (skinny_tail_on && force < 0 && a.groups_per_fold == 1 && whole > 0 && whole < n_tiles && planes_fit) {
         const int tail_panels = a.L.n_panels - whole / n_tok_tiles * 4;
         const int64_t wgs = (int64_t) tail_panels * ((a.M + 31) / 32);
         const double c = 2.6 * (whole / kCUs) + 0.65 * ((wgs + kCUs - 1) / kCUs);
