@@ -132,6 +132,10 @@ struct RotQuantArgs {
     int32_t      len_field;               // kActBlocks: pad[1] of the activation blocks (K or n_rot)
     float       *u;
     uint32_t    *act;                     // kActI8
+    // kActI8, single-plane form for the skinny kernel at 17..64 tokens: one int8 plane of q - z
+    // [g][quarter][Mp][16 bytes] at `act`, and the group multipliers m as bytes [g][Mp] at `mvals`
+    int          single;
+    uint8_t     *mvals;
     int          Mp;                      // kActI8: padded token count (rows M..Mp-1 are zero filled)
     // split-K scratch to clear (blocks past the token blocks do it)
     int32_t     *zero_ptr;
@@ -222,7 +226,8 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
 // up to 64 tokens: MFMA arithmetic on a GEMV-shaped weight stream; same operands as the GEMM plus the split-K cells
 struct SkinnyArgs {
     FusedWeights    w;
-    const uint8_t  *act8;   // [g][digit][quarter][Mp][16]
+    const uint8_t  *act8;   // [g][digit][quarter][Mp][16], or [g][quarter][Mp][16] with mvals (single plane)
+    const uint8_t  *mvals;  // null: two digit planes
     const float    *u;      // [Mp]
     int             M, Mp;
     int32_t        *tot;    // split-K cells [M][panels of all weights * 64], 64 bits each

@@ -191,6 +191,15 @@ __device__ __forceinline__ void digits_of_word(const float (&f)[8], float inv, f
     hi_o = pack_low_bytes(hi[1], hi[3], hi[5], hi[7]);
 }
 
+// Single-plane form: the bytes are q - z (-15 .. 15); the group multiplier travels beside the plane.
+__device__ __forceinline__ void qz_of_word(const float (&f)[8], float inv, float zf, uint32_t &even, uint32_t &odd) {
+    int d[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) d[j] = (int) (fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f) - zf);
+    even = pack_low_bytes(d[0], d[2], d[4], d[6]);
+    odd = pack_low_bytes(d[1], d[3], d[5], d[7]);
+}
+
 // Workgroup barrier for data that travels through LDS only: waits for this wavefront's LDS operations, not for its
 // outstanding global loads (which __syncthreads() would also drain, stalling a kernel that keeps weight loads in
 // flight across its prologue).

@@ -131,6 +131,14 @@ __global__ void __launch_bounds__(kRT) rq_quantize_digits_kernel(const RotQuantA
     const float4 *src = reinterpret_cast<const float4 *>(a.out_f32 + (int64_t) t * a.ldo + 8 * w);
     const float4 v0 = src[0], v1 = src[1];
     const float f[8] = { v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w };
+    if (a.single) {
+        uint32_t even, odd;
+        qz_of_word(f, inv, zf, even, odd);
+        const size_t cell1 = ((size_t) g * 4 + ((w & 7) >> 1)) * a.Mp + t;
+        *reinterpret_cast<uint2 *>(a.act + cell1 * 4 + (w & 1) * 2) = make_uint2(even, odd);
+        if ((w & 7) == 0) a.mvals[(size_t) g * a.Mp + t] = (uint8_t) mg;
+        return;
+    }
     uint32_t lo_e, lo_o, hi_e, hi_o;
     digits_of_word(f, inv, zf, (float) mg, lo_e, lo_o, hi_e, hi_o);
     // [group][digit][quarter of the group][token][16 bytes]

@@ -222,6 +222,17 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
         const int z = (int) zf;
         const float *sp = buf + padi(8 * wc);
         const float f[8] = { sp[0], sp[1], sp[2], sp[3], sp[4], sp[5], sp[6], sp[7] };
+        if (a.mode == kActI8 && a.single) {
+            uint32_t even, odd;
+            qz_of_word(f, inv, zf, even, odd);
+            if (on) {
+                // [group][quarter of the group][token][16 bytes] and the multiplier of (group, token)
+                const size_t cell = ((size_t) g * 4 + ((w & 7) >> 1)) * a.Mp + t;
+                *reinterpret_cast<uint2 *>(a.act + cell * 4 + (w & 1) * 2) = make_uint2(even, odd);
+                if ((w & 7) == 0) a.mvals[(size_t) g * a.Mp + t] = (uint8_t) mg;
+            }
+            continue;
+        }
         if (a.mode == kActI8) {
             uint32_t lo_e, lo_o, hi_e, hi_o;
             digits_of_word(f, inv, zf, (float) mg, lo_e, lo_o, hi_e, hi_o);

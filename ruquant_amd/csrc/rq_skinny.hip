@@ -39,10 +39,13 @@ __device__ __forceinline__ void widen(uint32_t w, int &even, int &odd) {
     odd = (int) (w & 0xF0F0F0F0u);
 }
 
-template <int TT>
+// SINGLE: the activations arrive as one plane of q - z plus the multiplier m of (group, token) as a byte (17..64
+// tokens: half the activation bytes per group); otherwise as the two digit planes of m (q - z).
+template <int TT, bool SINGLE>
 struct Frag {
-    uint2 a[4];        // packed weights of the four 16-row tiles: this lane's quarter of the group
-    uint4 b[TT][2];    // activation digits (lo, hi) of the token tiles: this lane's quarter
+    uint2 a[4];                  // packed weights of the four 16-row tiles: this lane's quarter of the group
+    uint4 b[TT][SINGLE ? 1 : 2]; // activation bytes of the token tiles: this lane's quarter
+    uint8_t mv[TT];              // SINGLE: multiplier of this lane's token
 };
 
 // Addresses are a uniform base (the panel's codes, the digit planes) plus a 32-bit offset per lane. `live` is uniform
@@ -50,29 +53,39 @@ struct Frag {
 // branch-free, so the wait counts stay exact) but with offset 0 in every lane, a few bytes that all lanes share:
 // memory throughput per compute unit is what bounds this kernel, and a ring that fetched real groups past the end
 // would add up to `depth` groups to every wavefront's share.
-template <int TT>
-__device__ __forceinline__ void load_frag(Frag<TT> &f, const uint8_t *a_panel, uint32_t a_lane, const uint8_t *b_planes,
-                                          uint32_t b_lane, int g, int Mp, bool live) {
+template <int TT, bool SINGLE>
+__device__ __forceinline__ void load_frag(Frag<TT, SINGLE> &f, const uint8_t *a_panel, uint32_t a_lane,
+                                          const uint8_t *b_planes, uint32_t b_lane, const uint8_t *mvals,
+                                          uint32_t m_lane, int g, int Mp, bool live) {
     // weights are read once (twice with two token blocks, and then from L2 at once): non-temporal, so they do not
-    // displace the digit planes, which every workgroup re-reads
+    // displace the activation planes, which every workgroup re-reads
     typedef unsigned v2u __attribute__((ext_vector_type(2)));
     const uint32_t ao = live ? a_lane + (uint32_t) g * 2048u : 0u;
-    const uint32_t bo = live ? b_lane + (uint32_t) g * 128u * (uint32_t) Mp : 0u;
+    const uint32_t bo = live ? b_lane + (uint32_t) g * (SINGLE ? 64u : 128u) * (uint32_t) Mp : 0u;
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
         const v2u v = __builtin_nontemporal_load(reinterpret_cast<const v2u *>(a_panel + ao + rt * 256));
         f.a[rt] = make_uint2(v.x, v.y);
     }
-    const uint32_t plane = 64u * (uint32_t) Mp;   // bytes from the low digits of a group to its high digits
+    if constexpr (SINGLE) {
+        const uint32_t mo = live ? m_lane + (uint32_t) g * (uint32_t) Mp : 0u;
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-        f.b[tt][0] = *reinterpret_cast<const uint4 *>(b_planes + bo + 256 * tt);
-        f.b[tt][1] = *reinterpret_cast<const uint4 *>(b_planes + bo + plane + 256 * tt);
+        for (int tt = 0; tt < TT; ++tt) {
+            f.b[tt][0] = *reinterpret_cast<const uint4 *>(b_planes + bo + 256 * tt);
+            f.mv[tt] = mvals[mo + 16 * tt];
+        }
+    } else {
+        const uint32_t plane = 64u * (uint32_t) Mp;   // bytes from the low digits of a group to its high digits
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+            f.b[tt][0] = *reinterpret_cast<const uint4 *>(b_planes + bo + 256 * tt);
+            f.b[tt][1] = *reinterpret_cast<const uint4 *>(b_planes + bo + plane + 256 * tt);
+        }
     }
 }
 
-template <int TT, bool HASK>
-__device__ __forceinline__ void mma_frag(const Frag<TT> &f, const uint8_t *k_base, int g, v4i (&hi)[4][TT],
+template <int TT, bool HASK, bool SINGLE>
+__device__ __forceinline__ void mma_frag(const Frag<TT, SINGLE> &f, const uint8_t *k_base, int g, v4i (&hi)[4][TT],
                                          int32_t (&lo)[4][TT][4]) {
     v4i A[4];
 #pragma unroll
@@ -94,19 +107,30 @@ __device__ __forceinline__ void mma_frag(const Frag<TT> &f, const uint8_t *k_bas
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
         const v4i Blo = v4i{ (int) f.b[tt][0].x, (int) f.b[tt][0].y, (int) f.b[tt][0].z, (int) f.b[tt][0].w };
-        const v4i Bhi = v4i{ (int) f.b[tt][1].x, (int) f.b[tt][1].y, (int) f.b[tt][1].z, (int) f.b[tt][1].w };
+        if constexpr (SINGLE) {
+            // S = 16 sum w (q - z); the group's term is floor(k m sum / 16) = (k m S) >> 8: |S| < 2^17, k m < 2^12
+            const int mg = (int) f.mv[tt];
 #pragma unroll
-        for (int rt = 0; rt < 4; ++rt) {
-            if (!HASK) {
-                hi[rt][tt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Bhi, hi[rt][tt], 0, 0, 0);
+            for (int rt = 0; rt < 4; ++rt) {
                 const v4i S = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Blo, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) lo[rt][tt][i] += S[i] >> 8;
-            } else {
-                const v4i H = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Bhi, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
-                const v4i S = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Blo, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+                for (int i = 0; i < 4; ++i) lo[rt][tt][i] += __mul24(S[i], HASK ? kk[rt][i] * mg : mg) >> 8;
+            }
+        } else {
+            const v4i Bhi = v4i{ (int) f.b[tt][1].x, (int) f.b[tt][1].y, (int) f.b[tt][1].z, (int) f.b[tt][1].w };
 #pragma unroll
-                for (int i = 0; i < 4; ++i) lo[rt][tt][i] += (kk[rt][i] * ((H[i] << 6) + S[i])) >> 8;
+            for (int rt = 0; rt < 4; ++rt) {
+                if (!HASK) {
+                    hi[rt][tt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Bhi, hi[rt][tt], 0, 0, 0);
+                    const v4i S = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Blo, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) lo[rt][tt][i] += S[i] >> 8;
+                } else {
+                    const v4i H = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Bhi, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+                    const v4i S = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], Blo, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) lo[rt][tt][i] += (kk[rt][i] * ((H[i] << 6) + S[i])) >> 8;
+                }
             }
         }
     }
@@ -116,18 +140,20 @@ __device__ __forceinline__ void mma_frag(const Frag<TT> &f, const uint8_t *k_bas
 // group j; the slot is refilled with group j + D as soon as group j's MFMAs have been issued. The scheduling
 // barriers keep the compiler from sinking those loads to their first use (which would expose the whole memory
 // latency once per group). Past the end the ring issues idle loads, and nothing consumes them.
-template <int TT>
-__device__ __forceinline__ void fill_ring(Frag<TT> (&ring)[depth_of(TT)], const uint8_t *a_panel, uint32_t a_lane,
-                                          const uint8_t *b_planes, uint32_t b_lane, int Mp, int g_first, int n) {
+template <int TT, bool SINGLE>
+__device__ __forceinline__ void fill_ring(Frag<TT, SINGLE> (&ring)[depth_of(TT)], const uint8_t *a_panel, uint32_t a_lane,
+                                          const uint8_t *b_planes, uint32_t b_lane, const uint8_t *mvals,
+                                          uint32_t m_lane, int Mp, int g_first, int n) {
 #pragma unroll
     for (int i = 0; i < depth_of(TT); ++i) {
-        load_frag<TT>(ring[i], a_panel, a_lane, b_planes, b_lane, g_first + i * kWaves, Mp, i < n);
+        load_frag<TT, SINGLE>(ring[i], a_panel, a_lane, b_planes, b_lane, mvals, m_lane, g_first + i * kWaves, Mp, i < n);
     }
 }
 
-template <int TT, bool HASK>
-__device__ __forceinline__ void stream_slice(Frag<TT> (&ring)[depth_of(TT)], const uint8_t *a_panel, uint32_t a_lane,
-                                             const uint8_t *b_planes, uint32_t b_lane, const uint8_t *k_base, int Mp,
+template <int TT, bool HASK, bool SINGLE>
+__device__ __forceinline__ void stream_slice(Frag<TT, SINGLE> (&ring)[depth_of(TT)], const uint8_t *a_panel,
+                                             uint32_t a_lane, const uint8_t *b_planes, uint32_t b_lane,
+                                             const uint8_t *mvals, uint32_t m_lane, const uint8_t *k_base, int Mp,
                                              int g_first, int n, v4i (&hi)[4][TT], int32_t (&lo)[4][TT][4]) {
     constexpr int D = depth_of(TT);
     // whole rounds of the ring: branch-free, so the wait counts before each group's MFMAs are exact
@@ -138,9 +164,9 @@ __device__ __forceinline__ void stream_slice(Frag<TT> (&ring)[depth_of(TT)], con
             const int j = r * D + i;
             const int g = g_first + j * kWaves;
             __builtin_amdgcn_sched_barrier(0);
-            mma_frag<TT, HASK>(ring[i], k_base, g, hi, lo);
+            mma_frag<TT, HASK, SINGLE>(ring[i], k_base, g, hi, lo);
             __builtin_amdgcn_sched_barrier(0);
-            load_frag<TT>(ring[i], a_panel, a_lane, b_planes, b_lane, g + D * kWaves, Mp, j + D < n);
+            load_frag<TT, SINGLE>(ring[i], a_panel, a_lane, b_planes, b_lane, mvals, m_lane, g + D * kWaves, Mp, j + D < n);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -148,13 +174,14 @@ __device__ __forceinline__ void stream_slice(Frag<TT> (&ring)[depth_of(TT)], con
     const int rem = n - rounds * D;
 #pragma unroll
     for (int i = 0; i < D - 1; ++i) {
-        if (i < rem) mma_frag<TT, HASK>(ring[i], k_base, g_first + (rounds * D + i) * kWaves, hi, lo);
+        if (i < rem) mma_frag<TT, HASK, SINGLE>(ring[i], k_base, g_first + (rounds * D + i) * kWaves, hi, lo);
     }
 }
 
-template <int TT>
-__global__ void __launch_bounds__(kThreads, TT == 1 ? 4 : 2)   // wavefronts per SIMD: two workgroups per CU at TT = 1
-rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const float *__restrict__ u, int M, int Mp,
+template <int TT, bool SINGLE>
+__global__ void __launch_bounds__(kThreads, TT == 1 ? 4 : SINGLE ? 3 : 2)   // wavefronts per SIMD: 4 = two workgroups per CU
+rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const uint8_t *__restrict__ mvals,
+                 const float *__restrict__ u, int M, int Mp,
                  int n_units, int nz,
                  unsigned long long *__restrict__ cells, int n_rows_pad, int main_panels, int tail_split,
                  int slice_base, int slice_extra, int panel0) {
@@ -209,6 +236,7 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const float
     // this lane's cell of the digit planes: quarter quad, token t0 + l16 (+ 16 per token tile)
     const uint8_t *b_planes = reinterpret_cast<const uint8_t *>(act8);
     const uint32_t b_lane = ((uint32_t) quad * Mp + t0 + l16) * 16u;
+    const uint32_t m_lane = (uint32_t) (t0 + l16);   // SINGLE: the multiplier of this lane's token (+ 16 per token tile)
     const uint8_t *k_base = kmul + (size_t) wpanel * ng * kPanelRows + 4 * quad;
 
     v4i hi[4][TT];
@@ -236,17 +264,17 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const float
     // the first loads go out before anything that waits (the LDS clear)
     const int g_first = g_begin + wave;
     const int n = g_first < g_end ? (g_end - g_first + kWaves - 1) / kWaves : 0;
-    Frag<TT> ring[depth_of(TT)];
-    fill_ring<TT>(ring, a_panel, a_lane, b_planes, b_lane, Mp, g_first, n);
+    Frag<TT, SINGLE> ring[depth_of(TT)];
+    fill_ring<TT, SINGLE>(ring, a_panel, a_lane, b_planes, b_lane, mvals, m_lane, Mp, g_first, n);
     __builtin_amdgcn_sched_barrier(0);
 
     for (int i = tid; i < 64 * kStride; i += kThreads) s_tot[i] = 0;
 
     if (n > 0) {
         if (has_k) {
-            stream_slice<TT, true>(ring, a_panel, a_lane, b_planes, b_lane, k_base, Mp, g_first, n, hi, lo);
+            stream_slice<TT, true, SINGLE>(ring, a_panel, a_lane, b_planes, b_lane, mvals, m_lane, k_base, Mp, g_first, n, hi, lo);
         } else {
-            stream_slice<TT, false>(ring, a_panel, a_lane, b_planes, b_lane, k_base, Mp, g_first, n, hi, lo);
+            stream_slice<TT, false, SINGLE>(ring, a_panel, a_lane, b_planes, b_lane, mvals, m_lane, k_base, Mp, g_first, n, hi, lo);
         }
     }
 
@@ -258,7 +286,7 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const float
         for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int32_t tot = (hi[rt][tt][i] >> 2) + lo[rt][tt][i];
+                const int32_t tot = SINGLE ? lo[rt][tt][i] : (hi[rt][tt][i] >> 2) + lo[rt][tt][i];
                 atomicAdd(&s_tot[(16 * rt + 4 * quad + i) * kStride + 16 * tt + l16], tot);
             }
         }
@@ -285,7 +313,7 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const float
     }
 }
 
-template <int TT>
+template <int TT, bool SINGLE>
 hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
     const WeightSet ws = make_weight_set(a.w);
     const int n_panels = a.panels > 0 ? a.panels : ws.first[kMaxFused];
@@ -299,8 +327,8 @@ hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
     }
     const int n_units = plan.main_panels + (n_panels - plan.main_panels) * plan.tail_split;
     const int blocks = (n_units + 7) / 8 * 8 * nz;
-    hipLaunchKernelGGL((rq_skinny_kernel<TT>), dim3(blocks), dim3(kThreads), 0, stream, ws,
-                       reinterpret_cast<const uint4 *>(a.act8), a.u, a.M, a.Mp, n_units, nz,
+    hipLaunchKernelGGL((rq_skinny_kernel<TT, SINGLE>), dim3(blocks), dim3(kThreads), 0, stream, ws,
+                       reinterpret_cast<const uint4 *>(a.act8), a.mvals, a.u, a.M, a.Mp, n_units, nz,
                        reinterpret_cast<unsigned long long *>(a.tot), ws.first[kMaxFused] * kPanelRows,
                        plan.main_panels, plan.tail_split, ws.ng / plan.tail_split, ws.ng % plan.tail_split,
                        a.panels > 0 ? a.panel0 : 0);
@@ -354,9 +382,10 @@ SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz) {
 
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream) {
     static const int tt1_max = getenv("RQ_SKINNY_TT1_MAX") ? atoi(getenv("RQ_SKINNY_TT1_MAX")) : 16;
-    if (a.panels > 0) return launch_tt<2>(a, stream);   // the tail of a GEMM launch: blocks of 32 tokens
-    if (a.M <= (tt1_max > 64 ? 64 : tt1_max)) return launch_tt<1>(a, stream);
-    return launch_tt<2>(a, stream);
+    if (a.panels > 0) return launch_tt<2, false>(a, stream);   // the tail of a GEMM launch: blocks of 32 tokens
+    if (a.mvals != nullptr) return launch_tt<2, true>(a, stream);   // the caller wrote single-plane activations
+    if (a.M <= (tt1_max > 64 ? 64 : tt1_max)) return launch_tt<1, false>(a, stream);
+    return launch_tt<2, false>(a, stream);
 }
 
 }  // namespace rq
