@@ -179,7 +179,7 @@ __device__ __forceinline__ void stream_slice(Frag<TT, SINGLE> (&ring)[depth_of(T
 }
 
 template <int TT, bool SINGLE>
-__global__ void __launch_bounds__(kThreads, TT == 1 ? 4 : SINGLE ? 3 : 2)   // wavefronts per SIMD: 4 = two workgroups per CU
+__global__ void __launch_bounds__(kThreads, TT == 1 ? 4 : (SINGLE && TT == 2) ? 3 : 2)   // wavefronts per SIMD: 4 = two workgroups per CU
 rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const uint8_t *__restrict__ mvals,
                  const float *__restrict__ u, int M, int Mp,
                  int n_units, int nz,
@@ -383,7 +383,18 @@ SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz) {
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream) {
     static const int tt1_max = getenv("RQ_SKINNY_TT1_MAX") ? atoi(getenv("RQ_SKINNY_TT1_MAX")) : 16;
     if (a.panels > 0) return launch_tt<2, false>(a, stream);   // the tail of a GEMM launch: blocks of 32 tokens
-    if (a.mvals != nullptr) return launch_tt<2, true>(a, stream);   // the caller wrote single-plane activations
+    if (a.mvals != nullptr) {   // the caller wrote single-plane activations
+        // 33..64 tokens: one workgroup with four token tiles per wavefront reads the weights once and halves the
+        // workgroup count, two blocks of 32 tokens give twice the workgroups. The former wins on long rows and on
+        // weights with a whole round of panels (K=17408, N=5120, M=64: 22.7 against 26.9 us; K=5120, N=17408: 27.1
+        // against 27.9), the latter on small weights (K=5120, N=5120: 10.9 against 15.8 us).
+        static const int wide_tokens = getenv("RQ_SKINNY_WIDE") ? atoi(getenv("RQ_SKINNY_WIDE")) : -1;
+        int n_panels = 0;
+        for (int i = 0; i < a.w.n; ++i) n_panels += a.w.L[i].n_panels;
+        const bool wide = wide_tokens >= 0 ? wide_tokens != 0 : (a.w.L[0].ng >= 160 || n_panels >= 256);
+        if (a.M > 32 && wide) return launch_tt<4, true>(a, stream);
+        return launch_tt<2, true>(a, stream);
+    }
     if (a.M <= (tt1_max > 64 ? 64 : tt1_max)) return launch_tt<1, false>(a, stream);
     return launch_tt<2, false>(a, stream);
 }
