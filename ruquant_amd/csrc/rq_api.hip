@@ -41,7 +41,7 @@ struct Env {
     int   act_group;
     int   gemm_min;  // smallest token count that takes the tiled MFMA GEMM
     int   gemv_max;  // largest token count that takes the GEMV; between the two: the skinny MFMA kernel
-    int   skinny_single;  // 17..64 tokens: single-plane activations (RQ_SKINNY_SINGLE=0 switches back to two digits)
+    int   skinny_single;  // skinny path: single-plane activations (RQ_SKINNY_SINGLE=0 switches back to two digits)
     Env() {
         const char *e = getenv("RQ_ACT_CLIP");
         const char *eh = getenv("RQ_ACT_CLIP_H");
@@ -156,9 +156,9 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     // plane would put all of its reads on the few L2 channels that the used 256 bytes of every 2 KB map to)
     const int act_mp = path == kPathSkinny ? (int) ((M + 15) / 16 * 16) : (int) W.Mp;
     q.Mp = act_mp;
-    // 17..64 tokens on the skinny path: one plane of q - z and the multipliers beside it (half the activation bytes
-    // per group, which at two token tiles per wavefront is what limits the workgroup's stream)
-    const bool single = path == kPathSkinny && M > 16 && env().skinny_single;
+    // the skinny path: one plane of q - z and the multipliers beside it (half the activation bytes per group, which
+    // count against the weight bytes a compute unit can have in flight)
+    const bool single = path == kPathSkinny && env().skinny_single;
     q.single = single;
     q.mvals = reinterpret_cast<uint8_t *>(wsb + W.off_i8) + (size_t) (K / kGroup) * act_mp * 64;
     const float *gemv_x = x;      // what the GEMV quantizes from: the rotated rows, or x itself for W4A4

@@ -132,7 +132,7 @@ struct RotQuantArgs {
     int32_t      len_field;               // kActBlocks: pad[1] of the activation blocks (K or n_rot)
     float       *u;
     uint32_t    *act;                     // kActI8
-    // kActI8, single-plane form for the skinny kernel at 17..64 tokens: one int8 plane of q - z
+    // kActI8, single-plane form for the skinny kernel: one int8 plane of q - z
     // [g][quarter][Mp][16 bytes] at `act`, and the group multipliers m as bytes [g][Mp] at `mvals`
     int          single;
     uint8_t     *mvals;

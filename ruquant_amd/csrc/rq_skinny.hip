@@ -39,8 +39,8 @@ __device__ __forceinline__ void widen(uint32_t w, int &even, int &odd) {
     odd = (int) (w & 0xF0F0F0F0u);
 }
 
-// SINGLE: the activations arrive as one plane of q - z plus the multiplier m of (group, token) as a byte (17..64
-// tokens: half the activation bytes per group); otherwise as the two digit planes of m (q - z).
+// SINGLE: the activations arrive as one plane of q - z plus the multiplier m of (group, token) as a byte (half the
+// activation bytes per group); otherwise as the two digit planes of m (q - z), which the GEMM's leftover rows use.
 template <int TT, bool SINGLE>
 struct Frag {
     uint2 a[4];                  // packed weights of the four 16-row tiles: this lane's quarter of the group
@@ -393,6 +393,7 @@ hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream) {
         for (int i = 0; i < a.w.n; ++i) n_panels += a.w.L[i].n_panels;
         const bool wide = wide_tokens >= 0 ? wide_tokens != 0 : (a.w.L[0].ng >= 160 || n_panels >= 256);
         if (a.M > 32 && wide) return launch_tt<4, true>(a, stream);
+        if (a.M <= 16) return launch_tt<1, true>(a, stream);
         return launch_tt<2, true>(a, stream);
     }
     if (a.M <= (tt1_max > 64 ? 64 : tt1_max)) return launch_tt<1, false>(a, stream);
