@@ -55,7 +55,7 @@ struct Env {
         if (gemm_min < 1) gemm_min = 1;
         if (gemm_min > kSkinnyTokens + 1) gemm_min = kSkinnyTokens + 1;
         const char *gv = getenv("RQ_GEMV_MAX");
-        gemv_max = gv ? atoi(gv) : 4;   // measured: from five tokens on the skinny MFMA kernel is the faster op
+        gemv_max = gv ? atoi(gv) : 3;   // measured: from four tokens on the skinny MFMA kernel is the faster op
         if (gemv_max < 0) gemv_max = 0;
         if (gemv_max > kGemvMaxTokens) gemv_max = kGemvMaxTokens;
         const char *ss = getenv("RQ_SKINNY_SINGLE");
