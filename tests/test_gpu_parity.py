@@ -354,6 +354,25 @@ def test_gemm_leftover_rows(oracle, N, M, wgroup):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
+@pytest.mark.parametrize("type_", [rq.TYPE_W4A4, rq.TYPE_W4A4H], ids=["w4a4", "w4a4h"])
+@pytest.mark.parametrize("M", [33, 50, 64])
+def test_skinny_all_tokens_in_one_workgroup_with_multipliers(oracle, M, type_):
+    """Long rows (K = 10240) at 33..64 tokens: the skinny kernel takes all tokens in one workgroup (four token tiles
+    per wavefront, single-plane activations); here with weight multipliers per 64 inputs and a partly filled panel."""
+    N, K = 200, 10240
+    rng = np.random.default_rng(M)
+    codes = rng.integers(-8, 8, size=(N, K), dtype=np.int8)
+    units = np.abs(rng.normal(0.02, 0.005, size=N)).astype(np.float32)
+    mults = rng.integers(1, 16, size=(N, K // 64), dtype=np.uint8)
+    b = rq.pack_groups(codes, units, mults)
+    rq.set_clip(b, 0.9)
+    W = rq.W4A4Weight(b, type_, DEV)
+    x = synth.activations("student_t4", M, K, 3 + M)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, b, x, W.clip, n_rot=K)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
 # ---------------------------------------------------------------- properties that hold at any size
 
 @pytest.mark.parametrize("M", [1, 8, 16, 200])
