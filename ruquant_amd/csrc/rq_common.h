@@ -16,6 +16,7 @@ constexpr int kGemvTokens = 8;    // tokens per GEMV pass; the activation slot s
 constexpr int kGemmTokens = 128;  // token tile of the MFMA GEMM; int8 activations are padded to it
 constexpr int kRangeParts = 32;    // partial maxima of a token's group ranges handed from the activation kernel to the GEMV
 constexpr int kSkinnyTokens = 64;   // most tokens of one pass of the skinny MFMA kernel
+constexpr int kTwoStepTokens = 40;   // long Paley stages: most tokens whose rotation is spread over several workgroups each
 constexpr int kGemvMaxTokens = 64;  // the dispatcher never sends more tokens than this down the GEMV path
 
 // ---------------------------------------------------------------------------------------------------

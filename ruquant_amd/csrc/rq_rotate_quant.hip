@@ -318,7 +318,8 @@ template <int P>
 hipError_t launch_p(const RotQuantArgs &a, hipStream_t stream) {
     const size_t row = (size_t) (a.K + (a.K >> 4) + 1) * sizeof(float);
     const size_t stats = (size_t) 2 * (a.K / kGroup + 1) * sizeof(float);
-    if (P > 1 && a.M <= 64 && 2 * row + stats <= 160 * 1024 - 64) {
+    // long Paley stages: past kTwoStepTokens tokens the plain variant (two workgroups per CU) is the faster one
+    if (P > 1 && a.M <= (P >= 44 ? kTwoStepTokens : 64) && 2 * row + stats <= 160 * 1024 - 64) {
         return launch_one<P, (P > 1)>(a, 2 * row + stats, stream);
     }
     return launch_one<P, false>(a, row + stats, stream);
