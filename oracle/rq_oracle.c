@@ -11,8 +11,12 @@
  * the same row search and code rule (int4_scale and code, src/gptq.rs:13-38, restated from the Rust text and
  * compared bit for bit), by the minimum property of the chosen ratio in exact rational arithmetic, by what the
  * reference's test asserts about weight groups (src/gptq.rs:303-311) and by round trips through the dequantizers
- * (tests/test_oracle_weight_quant.py). The activation dequantizers (rqo_dequantize_row_a) are pinned only through
- * those round-trip properties and the closed form of their one line: no reference-made value covers them.
+ * (tests/test_oracle_weight_quant.py). The activation dequantizers (rqo_dequantize_row_a) have no reference-made
+ * vector either; they are pinned by the reference's second statement of quantize-then-dequantize for grouped
+ * activations (fake_quant_groups, src/hessian.rs:70-92), restated from the Rust text: codes, zero points and
+ * multipliers must agree exactly, the values bit for bit under the C line's association (q - z) * (m * u) and
+ * within one unit in the last place under the Rust line's ((q - z) * m) * u; plus the rotation round trip for A4H
+ * (tests/test_oracle_act_dequant.py).
  *
  * Build: gcc -O3 -ffp-contract=off (no -ffast-math).
  */
