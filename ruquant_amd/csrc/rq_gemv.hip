@@ -141,6 +141,14 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
         pre_x1 = xp[1];
     }
 
+    // The epilogue's operands too (the row's scale, the weight's flag word): fetched at the end they would put one
+    // more trip to memory behind the last split-K arrival, on the critical path of the whole launch.
+    const float *__restrict__ s_w = wsel == 0 ? ws.s_w[0] : wsel == 1 ? ws.s_w[1] : ws.s_w[2];
+    const int64_t N = wsel == 0 ? ws.N[0] : wsel == 1 ? ws.N[1] : ws.N[2];
+    const int64_t n = (int64_t) wpanel * kPanelRows + lane;       // row of its weight
+    const float pre_sw = n < N ? s_w[n] : 0.0f;
+    const int32_t pre_flags = *reinterpret_cast<const volatile int32_t *>(flags);
+
     // ... and right behind them the weights of the first batch. This order matters: a wavefront's loads complete in
     // issue order, so the small prologue inputs must be the OLDER loads or they would wait for 10 KiB of weights.
     const uint4 *wp = codes + (size_t) wpanel * ng * 128 + lane;
@@ -200,7 +208,7 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
     had::lds_barrier();
 
     // ---- the product
-    const bool hask = *reinterpret_cast<const volatile int32_t *>(flags) & 1;
+    const bool hask = pre_flags & 1;
     int32_t tot[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) tot[t] = 0;
@@ -215,13 +223,10 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
     for (int t = 0; t < T; ++t) red[wave][t][lane] = tot[t];
     __syncthreads();
 
-    const float *__restrict__ s_w = wsel == 0 ? ws.s_w[0] : wsel == 1 ? ws.s_w[1] : ws.s_w[2];
     float *__restrict__ y = wsel == 0 ? ws.y[0] : wsel == 1 ? ws.y[1] : ws.y[2];
     const int64_t ldy = wsel == 0 ? ws.ldy[0] : wsel == 1 ? ws.ldy[1] : ws.ldy[2];
-    const int64_t N = wsel == 0 ? ws.N[0] : wsel == 1 ? ws.N[1] : ws.N[2];
     for (int item = tid; item < T * 64; item += NT) {
         const int t = item >> 6;
-        const int64_t n = (int64_t) wpanel * kPanelRows + lane;       // row of its weight
         const int64_t cell_row = (int64_t) panel * kPanelRows + lane;   // row of the launch (split-K cell)
         int32_t sum = 0;
 #pragma unroll
@@ -240,7 +245,7 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
             __hip_atomic_store(cell, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             sum = (int32_t) (uint32_t) now;  // the total fits int32 by construction of the format
         }
-        if (n < N) y[(int64_t) t * ldy + n] = (((float) sum * 16.0f) * s_u[t]) * s_w[n];
+        if (n < N) y[(int64_t) t * ldy + n] = (((float) sum * 16.0f) * s_u[t]) * pre_sw;
     }
 }
 
