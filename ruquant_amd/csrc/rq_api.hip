@@ -128,10 +128,11 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     if (ws_bytes < W.bytes || (reinterpret_cast<uintptr_t>(ws) & 255) != 0) return RQ_E_WORKSPACE;
     uint8_t *wsb = reinterpret_cast<uint8_t *>(ws);
 
-    // Activation groups of 128 / 256 (RQ_ACT_GROUP) change where the per-group floor falls; only the narrow-tile
-    // MFMA kernel folds at that granularity, so every token count takes it (a format variant, not a tuned path).
+    // Activation groups of 128 / 256 (RQ_ACT_GROUP) change where the per-group floor falls. The GEMV folds at that
+    // granularity for up to kGemvWideTokens tokens (decode); beyond that only the narrow-tile MFMA kernel does, so
+    // every larger token count takes it (a format variant, not a tuned path).
     const int G = env().act_group;
-    const Path path = G != 64 ? kPathGemm : path_of(M);
+    const Path path = G != 64 && !(path_of(M) == kPathGemv && M <= kGemvWideTokens) ? kPathGemm : path_of(M);
     const bool gemm = path != kPathGemv;   // the int8 digit planes feed both MFMA kernels
     RotQuantArgs q;
     memset(&q, 0, sizeof q);
@@ -145,7 +146,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     q.m = m;
     q.scale = 1.0f / sqrtf((float) q.n_rot);
     q.clip = clip;
-    q.G = G;
+    q.G = G;   // (the GEMV path takes ranges per run of 64 whatever G is, and folds them itself: set below)
     // Skinny batches with a long Paley stage: one workgroup per token would leave most of the chip idle for tens of
     // microseconds, so the rotation runs spread over workgroups (ranges out) and a second small kernel quantizes.
     // (up to 40 tokens: from there on the one-workgroup-per-token kernel has enough tokens to fill the chip: K = 17408,
@@ -165,6 +166,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     q.mvals = reinterpret_cast<uint8_t *>(wsb + W.off_i8) + (size_t) (K / kGroup) * act_mp * 64;
     const float *gemv_x = x;      // what the GEMV quantizes from: the rotated rows, or x itself for W4A4
     int64_t gemv_ldx = ldx;
+    if (!gemm) q.G = kGroup;
     if (!gemm || two_step) {
         q.lohi = reinterpret_cast<float *>(wsb + W.off_lohi);
         q.rpart = reinterpret_cast<float *>(wsb + W.off_rpart);
@@ -244,6 +246,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
                 g.lohi = q.lohi + (size_t) c * kGemvTokens * fw.L[0].ng * 2;
                 g.rpart = q.rpart + (size_t) c * kGemvTokens * kRangeParts;
                 g.T = (int) (M - (int64_t) c * kGemvTokens < kGemvTokens ? M - (int64_t) c * kGemvTokens : kGemvTokens);
+                g.gf = G / kGroup;
                 g.tot = reinterpret_cast<int32_t *>(wsb + W.off_tot);
                 e = launch_gemv(g, stream);
                 if (e != hipSuccess) return (int) e;

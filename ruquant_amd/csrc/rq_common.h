@@ -17,6 +17,7 @@ constexpr int kGemmTokens = 128;  // token tile of the MFMA GEMM; int8 activatio
 constexpr int kRangeParts = 32;    // partial maxima of a token's group ranges handed from the activation kernel to the GEMV
 constexpr int kSkinnyTokens = 64;   // most tokens of one pass of the skinny MFMA kernel
 constexpr int kTwoStepTokens = 40;   // long Paley stages: most tokens whose rotation is spread over several workgroups each
+constexpr int kGemvWideTokens = 3;   // most tokens of a GEMV pass with activation groups of 128 / 256
 constexpr int kGemvMaxTokens = 64;  // the dispatcher never sends more tokens than this down the GEMV path
 
 // ---------------------------------------------------------------------------------------------------
@@ -207,6 +208,7 @@ struct GemvArgs {
     const float    *lohi;   // clipped group ranges of this chunk's first token, [T][ng][2]
     const float    *rpart;  // partial range maxima of this chunk's first token, [T][kRangeParts]
     int             T;      // 1..8 tokens
+    int             gf;     // runs of 64 per activation group: 1, or 2 / 4 under RQ_ACT_GROUP (then T <= kGemvWideTokens)
     int32_t        *tot;    // split-K cells (zero on entry, left zero)
 };
 hipError_t launch_gemv(const GemvArgs &a, hipStream_t stream);

@@ -39,15 +39,23 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Activation groups wider than 64 (GF = 2 or 4 runs of 64 per group): a group's runs share one multiplier and zero
+// point and are folded once, so a wavefront takes whole groups ("units"). A batch is U runs of 64 per wavefront.
+template <int GF>
+constexpr int batch_runs() { return GF == 1 ? kUnroll : 4; }
+
+template <int U>
 struct Batch {
-    uint4 q[kUnroll][2];
+    uint4 q[U][2];
 };
 
-template <int kWaves>
-__device__ __forceinline__ void load_batch(Batch &b, const uint4 *wp, int g0, int g_end) {
+// u0: this wavefront's first unit of the batch; its next ones are kWaves units further on
+template <int kWaves, int U, int GF>
+__device__ __forceinline__ void load_batch(Batch<U> &b, const uint4 *wp, int u0, int u_end) {
 #pragma unroll
-    for (int k = 0; k < kUnroll; ++k) {
-        const int g = min(g0 + k * kWaves, g_end - 1);  // past the end: reread the last group, contribute nothing
+    for (int k = 0; k < U; ++k) {
+        const int u = min(u0 + (k / GF) * kWaves, u_end - 1);  // past the end: reread the last unit, contribute nothing
+        const int g = u * GF + k % GF;
         // weights are read once per call: non-temporal, so they do not displace the activations and ranges in L2
         typedef unsigned v4u __attribute__((ext_vector_type(4)));
         const v4u q0 = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(wp + (size_t) g * 128));
@@ -57,46 +65,58 @@ __device__ __forceinline__ void load_batch(Batch &b, const uint4 *wp, int g0, in
     }
 }
 
-// act: [group of the slice][token][8 words] codes q - 8 in the tensor's nibble order; mz: m | (8 - z) << 8
-template <int T, int kWaves>
-__device__ __forceinline__ void compute_batch(const Batch &b, const uint8_t *kp, bool hask, const uint32_t *act,
-                                              const int32_t *mz, int g0, int g_begin, int g_end, int32_t (&tot)[T]) {
+// act: [run of 64 of the slice][token][8 words] codes q - 8 in the tensor's nibble order; mz: [unit of the slice][token]
+// m | (8 - z) << 8. The weight multiplier of a unit is that of its first run (reference patch line 168).
+template <int T, int kWaves, int U, int GF>
+__device__ __forceinline__ void compute_batch(const Batch<U> &b, const uint8_t *kp, bool hask, const uint32_t *act,
+                                              const int32_t *mz, int u0, int u_begin, int u_end, int32_t (&tot)[T]) {
 #pragma unroll
-    for (int k = 0; k < kUnroll; ++k) {
-        const int g = g0 + k * kWaves;
-        if (g >= g_end) break;   // wave-uniform
-        const uint32_t w[8] = { b.q[k][0].x, b.q[k][0].y, b.q[k][0].z, b.q[k][0].w,
-                                b.q[k][1].x, b.q[k][1].y, b.q[k][1].z, b.q[k][1].w };
-        int cs = 0;
+    for (int j = 0; j < U / GF; ++j) {
+        const int u = u0 + j * kWaves;
+        if (u >= u_end) break;   // wave-uniform
+        const int ul = u - u_begin;
+        int part[T];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) cs = dot8(w[i], 0x11111111u, cs);
+        for (int t = 0; t < T; ++t) part[t] = 0;
+#pragma unroll
+        for (int sub = 0; sub < GF; ++sub) {
+            const int k = j * GF + sub;
+            const uint32_t w[8] = { b.q[k][0].x, b.q[k][0].y, b.q[k][0].z, b.q[k][0].w,
+                                    b.q[k][1].x, b.q[k][1].y, b.q[k][1].z, b.q[k][1].w };
+            int cs = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) cs = dot8(w[i], 0x11111111u, cs);
+            const int gl = ul * GF + sub;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const uint4 a0 = *reinterpret_cast<const uint4 *>(act + (gl * T + t) * 8);      // same address in every lane
+                const uint4 a1 = *reinterpret_cast<const uint4 *>(act + (gl * T + t) * 8 + 4);
+                int acc = 0;
+                acc = dot8(w[0], a0.x, acc);
+                acc = dot8(w[1], a0.y, acc);
+                acc = dot8(w[2], a0.z, acc);
+                acc = dot8(w[3], a0.w, acc);
+                acc = dot8(w[4], a1.x, acc);
+                acc = dot8(w[5], a1.y, acc);
+                acc = dot8(w[6], a1.z, acc);
+                acc = dot8(w[7], a1.w, acc);
+                const int zc = (int) (int8_t) ((mz[ul * T + t] >> 8) & 0xFF);
+                part[t] += acc + zc * cs;
+            }
+        }
         int kw = 1;
-        if (hask) kw = kp[(size_t) g * kPanelRows];
-        const int gl = g - g_begin;
+        if (hask) kw = kp[(size_t) (u * GF) * kPanelRows];
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-            const uint4 a0 = *reinterpret_cast<const uint4 *>(act + (gl * T + t) * 8);      // same address in every lane
-            const uint4 a1 = *reinterpret_cast<const uint4 *>(act + (gl * T + t) * 8 + 4);
-            int acc = 0;
-            acc = dot8(w[0], a0.x, acc);
-            acc = dot8(w[1], a0.y, acc);
-            acc = dot8(w[2], a0.z, acc);
-            acc = dot8(w[3], a0.w, acc);
-            acc = dot8(w[4], a1.x, acc);
-            acc = dot8(w[5], a1.y, acc);
-            acc = dot8(w[6], a1.z, acc);
-            acc = dot8(w[7], a1.w, acc);
-            const int32_t mzv = mz[gl * T + t];
-            const int mult = mzv & 0xFF;
-            const int zc = (int) (int8_t) ((mzv >> 8) & 0xFF);
-            int term = mult * (acc + zc * cs);
+            int term = (mz[ul * T + t] & 0xFF) * part[t];
             if (hask) term *= kw;
             tot[t] += term >> kTermShift;
         }
     }
 }
 
-template <int T, int kWaves>
+// slice_base / slice_extra: the split of K in units (activation groups)
+template <int T, int kWaves, int GF>
 __global__ void __launch_bounds__(kWaves * 64)
 rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, const float *__restrict__ lohi,
                const float *__restrict__ rpart, unsigned long long *__restrict__ cells, int n_rows_pad, int slice_base,
@@ -117,21 +137,24 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
     const uint4 *__restrict__ codes = reinterpret_cast<const uint4 *>(wsel == 0 ? ws.codes[0] : wsel == 1 ? ws.codes[1] : ws.codes[2]);
     const uint8_t *__restrict__ kmul = wsel == 0 ? ws.kmul[0] : wsel == 1 ? ws.kmul[1] : ws.kmul[2];
     const int32_t *__restrict__ flags = wsel == 0 ? ws.flags[0] : wsel == 1 ? ws.flags[1] : ws.flags[2];
+    constexpr int U = batch_runs<GF>();
     const int ng = ws.ng;
     const int nks = gridDim.y, ks = blockIdx.y;
-    // slices of ng / nks groups, the first ng % nks one longer (no division on the device)
-    const int g_begin = ks * slice_base + (ks < slice_extra ? ks : slice_extra);
-    const int g_end = g_begin + slice_base + (ks < slice_extra ? 1 : 0);
+    // slices of nu / nks units, the first nu % nks one longer (no division on the device)
+    const int u_begin = ks * slice_base + (ks < slice_extra ? ks : slice_extra);
+    const int u_end = u_begin + slice_base + (ks < slice_extra ? 1 : 0);
+    const int g_begin = u_begin * GF, g_end = u_end * GF;   // the same in runs of 64
     const int cnt = g_end - g_begin;
 
     // The three inputs of the quantizer prologue do not depend on each other: fetch this thread's share of all of
     // them first (partial range maxima, its first (group, token) range, its first code word's eight values), so the
     // prologue pays one memory latency, not three in a row.
-    const int n_gt = cnt * T, n_words = n_gt * 8;
+    const int n_ut = (u_end - u_begin) * T;        // (unit, token) pairs of the slice
+    const int n_words = cnt * T * 8;               // code words of the slice
     float pre_r = 0.0f;
-    if (tid < T * 64 && lane < kRangeParts) pre_r = rpart[(tid >> 6) * kRangeParts + lane];
+    if (GF == 1 && tid < T * 64 && lane < kRangeParts) pre_r = rpart[(tid >> 6) * kRangeParts + lane];
     float2 pre_lh = make_float2(0.0f, 0.0f);
-    if (tid < n_gt) pre_lh = reinterpret_cast<const float2 *>(lohi)[(size_t) (tid % T) * ng + g_begin + tid / T];
+    if (GF == 1 && tid < n_ut) pre_lh = reinterpret_cast<const float2 *>(lohi)[(size_t) (tid % T) * ng + g_begin + tid / T];
     float4 pre_x0 = make_float4(0.f, 0.f, 0.f, 0.f), pre_x1 = pre_x0;
     if (tid < n_words) {
         const int gt = tid >> 3;
@@ -153,14 +176,30 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
     // issue order, so the small prologue inputs must be the OLDER loads or they would wait for 10 KiB of weights.
     const uint4 *wp = codes + (size_t) wpanel * ng * 128 + lane;
     const uint8_t *kp = kmul + (size_t) wpanel * ng * kPanelRows + lane;
-    Batch b0;
-    load_batch<kWaves>(b0, wp, g_begin + wave, g_end);
+    Batch<U> b0;
+    load_batch<kWaves, U, GF>(b0, wp, u_begin + wave, u_end);
 
     // ---- token units: R = widest clipped group range of the whole token (the activation kernel left 32 partial
     // maxima per token), 2 if the token is all zero; u = R / 3825
     if (tid < T * 64) {
         for (int tt = tid >> 6; tt < T; tt += kWaves) {   // wavefront w handles tokens w, w + kWaves, ...
-            float r = tt == (tid >> 6) ? pre_r : (lane < kRangeParts ? rpart[tt * kRangeParts + lane] : 0.0f);
+            float r = 0.0f;
+            if constexpr (GF == 1) {
+                r = tt == (tid >> 6) ? pre_r : (lane < kRangeParts ? rpart[tt * kRangeParts + lane] : 0.0f);
+            } else {
+                // wide groups: the partial maxima are those of the runs of 64; the token's widest *group* comes from
+                // the runs' ranges (min and max commute with the multiplication by the positive clip)
+                for (int u = lane; u < ng / GF; u += 64) {
+                    float2 c = reinterpret_cast<const float2 *>(lohi)[(size_t) tt * ng + u * GF];
+#pragma unroll
+                    for (int sub = 1; sub < GF; ++sub) {
+                        const float2 o = reinterpret_cast<const float2 *>(lohi)[(size_t) tt * ng + u * GF + sub];
+                        c.x = fminf(c.x, o.x);
+                        c.y = fmaxf(c.y, o.y);
+                    }
+                    r = fmaxf(r, c.y - c.x);
+                }
+            }
             r = wave_max(r);
             if (r == 0.0f) r = 2.0f;
             if (lane == 0) {
@@ -172,9 +211,15 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
     had::lds_barrier();   // not __syncthreads(): the weight loads stay in flight across the prologue
 
     // ---- per (group of the slice, token): multiplier, 1 / (m u), zero point (reference lines 2662-2665)
-    for (int gt = tid; gt < n_gt; gt += NT) {
-        const int t = gt % T, g = g_begin + gt / T;
-        const float2 r = gt == tid ? pre_lh : reinterpret_cast<const float2 *>(lohi)[(size_t) t * ng + g];
+    for (int gt = tid; gt < n_ut; gt += NT) {
+        const int t = gt % T, g = (u_begin + gt / T) * GF;
+        float2 r = GF == 1 && gt == tid ? pre_lh : reinterpret_cast<const float2 *>(lohi)[(size_t) t * ng + g];
+#pragma unroll
+        for (int sub = 1; sub < GF; ++sub) {
+            const float2 o = reinterpret_cast<const float2 *>(lohi)[(size_t) t * ng + g + sub];
+            r.x = fminf(r.x, o.x);
+            r.y = fmaxf(r.y, o.y);
+        }
         const float lo = r.x, hi = r.y;
         const int mg = (int) fminf(fmaxf(ceilf(((hi - lo) * 255.0f) / s_R[t]), 1.0f), 255.0f);
         const float inv = 1.0f / ((float) mg * s_u[t]);
@@ -189,7 +234,8 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
     for (int id = tid; id < n_words; id += NT) {
         const int wi = id & 7, gt = id >> 3;
         const int t = gt % T, g = g_begin + gt / T;
-        const float inv = s_inv[gt], zf = s_zf[gt];
+        const int ut = (gt / T / GF) * T + t;     // its (unit, token) pair
+        const float inv = s_inv[ut], zf = s_zf[ut];
         float4 v0 = pre_x0, v1 = pre_x1;
         if (id != tid) {
             const float4 *xp = reinterpret_cast<const float4 *>(x + (int64_t) t * ldx + (int64_t) g * kGroup + wi * 8);
@@ -212,11 +258,11 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
     int32_t tot[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) tot[t] = 0;
-    compute_batch<T, kWaves>(b0, kp, hask, s_act, s_mz, g_begin + wave, g_begin, g_end, tot);
-    for (int g0 = g_begin + wave + kWaves * kUnroll; g0 < g_end; g0 += kWaves * kUnroll) {
-        Batch b;
-        load_batch<kWaves>(b, wp, g0, g_end);
-        compute_batch<T, kWaves>(b, kp, hask, s_act, s_mz, g0, g_begin, g_end, tot);
+    compute_batch<T, kWaves, U, GF>(b0, kp, hask, s_act, s_mz, u_begin + wave, u_begin, u_end, tot);
+    for (int u0 = u_begin + wave + kWaves * (U / GF); u0 < u_end; u0 += kWaves * (U / GF)) {
+        Batch<U> b;
+        load_batch<kWaves, U, GF>(b, wp, u0, u_end);
+        compute_batch<T, kWaves, U, GF>(b, kp, hask, s_act, s_mz, u0, u_begin, u_end, tot);
     }
 
 #pragma unroll
@@ -249,23 +295,30 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
     }
 }
 
-template <int T, int kWaves>
-hipError_t launch_tw(const GemvArgs &a, int nks, hipStream_t stream) {
+template <int T, int kWaves, int GF>
+hipError_t launch_twg(const GemvArgs &a, int nks, hipStream_t stream) {
     const WeightSet ws = make_weight_set(a.w);
     const int n_panels = ws.first[kMaxFused];
-    hipLaunchKernelGGL((rq_gemv_kernel<T, kWaves>), dim3(n_panels, nks), dim3(kWaves * 64), 0, stream, ws, a.x, a.ldx,
+    const int nu = ws.ng / GF;
+    hipLaunchKernelGGL((rq_gemv_kernel<T, kWaves, GF>), dim3(n_panels, nks), dim3(kWaves * 64), 0, stream, ws, a.x, a.ldx,
                        a.lohi, a.rpart, reinterpret_cast<unsigned long long *>(a.tot), n_panels * kPanelRows,
-                       ws.ng / nks, ws.ng % nks);
+                       nu / nks, nu % nks);
     return hipGetLastError();
 }
 
 template <int T>
 hipError_t launch_t(const GemvArgs &a, int nks, hipStream_t stream) {
     static const int waves = getenv("RQ_GEMV_WAVES") ? atoi(getenv("RQ_GEMV_WAVES")) : kGemvWaves;
+    if constexpr (T <= kGemvWideTokens) {
+        // activation groups of 128 / 256 (a format variant): one configuration
+        if (a.gf == 2) return launch_twg<T, kGemvWaves, 2>(a, nks, stream);
+        if (a.gf == 4) return launch_twg<T, kGemvWaves, 4>(a, nks, stream);
+    }
+    if (a.gf != 1) return hipErrorInvalidValue;
     switch (waves) {
-        case 2:  return launch_tw<T, 2>(a, nks, stream);
-        case 8:  return launch_tw<T, 8>(a, nks, stream);
-        default: return launch_tw<T, 4>(a, nks, stream);
+        case 2:  return launch_twg<T, 2, 1>(a, nks, stream);
+        case 8:  return launch_twg<T, 8, 1>(a, nks, stream);
+        default: return launch_twg<T, 4, 1>(a, nks, stream);
     }
 }
 
@@ -298,7 +351,15 @@ int gemv_ksplit(int n_panels, int ng) {
 hipError_t launch_gemv(const GemvArgs &a, hipStream_t stream) {
     int n_panels = 0;
     for (int i = 0; i < a.w.n; ++i) n_panels += a.w.L[i].n_panels;
-    const int nks = gemv_ksplit(n_panels, a.w.L[0].ng);
+    const int ng = a.w.L[0].ng;
+    int nks = gemv_ksplit(n_panels, ng);
+    if (a.gf > 1) {
+        // whole groups per slice, and no slice longer than the LDS of a workgroup holds
+        const int nu = ng / a.gf;
+        if (ng % a.gf != 0) return hipErrorInvalidValue;
+        if (nks > nu) nks = nu;
+        while (nks < nu && (nu + nks - 1) / nks * a.gf > kMaxSlice) ++nks;
+    }
     switch (a.T) {
         case 1: return launch_t<1>(a, nks, stream);
         case 2: return launch_t<2>(a, nks, stream);
