@@ -318,7 +318,7 @@ def main():
                    "algorithmic_bytes": b},
         "roofline": {"bound": "hbm", "achieved": round(b / kern_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(b / kern_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": HEADLINE_TRAFFIC_BYTES,
-                     "kernel": "rq_gemv_kernel<1, 4>", "kernel_us": round(kern_ms * 1e3, 3)},
+                     "kernel": "rq_gemv_kernel<1, 4, 1>", "kernel_us": round(kern_ms * 1e3, 3)},
         "cpu_baseline": cpu,
         "parity_vs_oracle": parity,
         "extra": extra,
