@@ -129,10 +129,11 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     uint8_t *wsb = reinterpret_cast<uint8_t *>(ws);
 
     // Activation groups of 128 / 256 (RQ_ACT_GROUP) change where the per-group floor falls. The GEMV folds at that
-    // granularity for up to kGemvWideTokens tokens (decode); beyond that only the narrow-tile MFMA kernel does, so
-    // every larger token count takes it (a format variant, not a tuned path).
+    // granularity for up to kGemvWideTokens tokens (one token 16 us, eight 33 us at K = 5120, N = 17408); beyond
+    // that only the narrow-tile MFMA kernel does (44 us from 4 to 64 tokens), so every larger token count takes it
+    // (a format variant, not a tuned path).
     const int G = env().act_group;
-    const Path path = G != 64 && !(path_of(M) == kPathGemv && M <= kGemvWideTokens) ? kPathGemm : path_of(M);
+    const Path path = G != 64 ? (M <= kGemvWideTokens ? kPathGemv : kPathGemm) : path_of(M);
     const bool gemm = path != kPathGemv;   // the int8 digit planes feed both MFMA kernels
     RotQuantArgs q;
     memset(&q, 0, sizeof q);

@@ -17,7 +17,7 @@ constexpr int kGemmTokens = 128;  // token tile of the MFMA GEMM; int8 activatio
 constexpr int kRangeParts = 32;    // partial maxima of a token's group ranges handed from the activation kernel to the GEMV
 constexpr int kSkinnyTokens = 64;   // most tokens of one pass of the skinny MFMA kernel
 constexpr int kTwoStepTokens = 40;   // long Paley stages: most tokens whose rotation is spread over several workgroups each
-constexpr int kGemvWideTokens = 3;   // most tokens of a GEMV pass with activation groups of 128 / 256
+constexpr int kGemvWideTokens = 8;   // most tokens of a GEMV pass with activation groups of 128 / 256
 constexpr int kGemvMaxTokens = 64;  // the dispatcher never sends more tokens than this down the GEMV path
 
 // ---------------------------------------------------------------------------------------------------

@@ -24,7 +24,7 @@ cases = [(rq.TYPE_W4A4H, 200, 1536, 0), (rq.TYPE_W4A4H, 200, 1536, 64), (rq.TYPE
 for type_, N, K, wgroup in cases:
     blocks, wf = adversarial_weights(rq_oracle, N, K, type_, wgroup=wgroup)
     W = rq.W4A4Weight(blocks, type_, DEV)
-    for M in (1, 2, 3, 40, 130):   # up to three tokens: the GEMV folds the wide groups; beyond: the narrow-tile GEMM
+    for M in (1, 2, 3, 5, 8, 9, 40, 130):   # up to eight tokens: the GEMV folds the wide groups; beyond: the narrow-tile GEMM
         x = adversarial_activations(M, K, type_, wf, seed=M)
         got = run_gpu(W, x)
         want = rq_oracle.mul_mat(type_, blocks, x, W.clip, n_rot=max(W.n_rot, 0), G=G)
