@@ -239,26 +239,42 @@ __device__ __forceinline__ void load_row(float *buf, const float *__restrict__ x
 // The row from global memory through the first four Sylvester stages (strides 1, 2, 4, 8; chunks of at least 16
 // floats) into the padded LDS row: a thread takes 16 consecutive floats, so the stages run in registers on the way in
 // and the row makes one trip through LDS less (worth 10-15 % of the kernel for one token and for thousands).
-template <int NT>
+// BATCH units per thread are requested before the first is worked on: a long row is several units per thread, and
+// taken one at a time each would cost a full trip to memory.
+template <int NT, int BATCH = 1>
 __device__ __forceinline__ void load_row_fwht16(float *buf, const float *__restrict__ xr, int K, int tid) {
-    for (int u = tid; u < (K >> 4); u += NT) {
-        const float4 *src = reinterpret_cast<const float4 *>(xr + 16 * u);
-        const float4 q0 = src[0], q1 = src[1], q2 = src[2], q3 = src[3];
-        float v[16] = { q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w, q2.x, q2.y, q2.z, q2.w, q3.x, q3.y, q3.z, q3.w };
+    for (int u0 = tid; u0 < (K >> 4); u0 += NT * BATCH) {
+        float4 q[BATCH][4];
 #pragma unroll
-        for (int h = 1; h < 16; h <<= 1) {
+        for (int b = 0; b < BATCH; ++b) {
+            const int u = u0 + b * NT;
+            if (u < (K >> 4)) {
+                const float4 *src = reinterpret_cast<const float4 *>(xr + 16 * u);
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                if ((j & h) == 0) {
-                    const float lo = v[j], up = v[j + h];
-                    v[j] = lo + up;
-                    v[j + h] = lo - up;
-                }
+                for (int j = 0; j < 4; ++j) q[b][j] = src[j];
             }
         }
-        float *d = buf + padi(16 * u);   // a run of 16 is contiguous in the padded row
 #pragma unroll
-        for (int j = 0; j < 16; ++j) d[j] = v[j];
+        for (int b = 0; b < BATCH; ++b) {
+            const int u = u0 + b * NT;
+            if (u >= (K >> 4)) break;
+            float v[16] = { q[b][0].x, q[b][0].y, q[b][0].z, q[b][0].w, q[b][1].x, q[b][1].y, q[b][1].z, q[b][1].w,
+                            q[b][2].x, q[b][2].y, q[b][2].z, q[b][2].w, q[b][3].x, q[b][3].y, q[b][3].z, q[b][3].w };
+#pragma unroll
+            for (int h = 1; h < 16; h <<= 1) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    if ((j & h) == 0) {
+                        const float lo = v[j], up = v[j + h];
+                        v[j] = lo + up;
+                        v[j + h] = lo - up;
+                    }
+                }
+            }
+            float *d = buf + padi(16 * u);   // a run of 16 is contiguous in the padded row
+#pragma unroll
+            for (int j = 0; j < 16; ++j) d[j] = v[j];
+        }
     }
 }
 

@@ -68,7 +68,9 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
     // the first four Sylvester stages ride on the load (one trip through LDS less per token)
     const bool fused_first = a.rotate && (a.m & 15) == 0;
     if (fused_first) {
-        load_row_fwht16<kNT>(buf, xr, K, tid);
+        // long Paley stages go with long rows (several units of 16 floats per thread): all of a thread's loads go
+        // out before the first butterfly
+        load_row_fwht16<kNT, (P >= 44 ? 3 : 1)>(buf, xr, K, tid);
     } else {
         load_row<kNT>(buf, xr, K, tid);
     }
