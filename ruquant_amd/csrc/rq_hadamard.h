@@ -126,6 +126,22 @@ __device__ __forceinline__ float wave_reduce(float v) {
 #undef RQ_DPP_STEP
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+// max / min over aligned runs of eight lanes, the same value in all eight
+template <bool MAX>
+__device__ __forceinline__ float group8_reduce(float v) {
+#define RQ_DPP_STEP(ctrl)                                                                                        \
+    {                                                                                                            \
+        const float o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v),         \
+                                                                              __builtin_bit_cast(int, v), ctrl,  \
+                                                                              0xF, 0xF, false));                 \
+        v = MAX ? fmaxf(v, o) : fminf(v, o);                                                                     \
+    }
+    RQ_DPP_STEP(0xB1)    // quad_perm [1, 0, 3, 2]
+    RQ_DPP_STEP(0x4E)    // quad_perm [2, 3, 0, 1]
+    RQ_DPP_STEP(0x141)   // row_half_mirror: lane i of a half row takes lane 7 - i, which sits in the other quad
+#undef RQ_DPP_STEP
+    return v;
+}
 __device__ __forceinline__ float wave_max(float v) { return wave_reduce<true>(v); }
 __device__ __forceinline__ float wave_min(float v) { return wave_reduce<false>(v); }
 

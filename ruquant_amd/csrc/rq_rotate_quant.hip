@@ -169,9 +169,16 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
             mn = fminf(fminf(fminf(fminf(mn, v0.x), fminf(v0.y, v0.z)), fminf(fminf(v0.w, v1.x), fminf(v1.y, v1.z))), v1.w);
             mx = fmaxf(fmaxf(fmaxf(fmaxf(mx, v0.x), fmaxf(v0.y, v0.z)), fmaxf(fmaxf(v0.w, v1.x), fmaxf(v1.y, v1.z))), v1.w);
         }
-        for (int off = 1; off < lpg; off <<= 1) {
-            mn = fminf(mn, __shfl_xor(mn, off, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        if (lpg == 8) {
+            // groups of 64 = eight lanes: swap within pairs, within quads, mirror the half row; DPP steps at vector-ALU
+            // speed instead of three trips through the LDS crossbar
+            mn = had::group8_reduce<false>(mn);
+            mx = had::group8_reduce<true>(mx);
+        } else {
+            for (int off = 1; off < lpg; off <<= 1) {
+                mn = fminf(mn, __shfl_xor(mn, off, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+            }
         }
         const float lo = mn * a.clip, hi = mx * a.clip;
         if (on) {
