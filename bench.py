@@ -199,7 +199,7 @@ class Layer:
                 "layer_us_seven_separate_calls": round(plain_ms * 1e3, 2)}
 
 
-def cpu_baseline(oracle, prob, budget_s=12.0, max_reps=400):
+def cpu_baseline(oracle, prob, budget_s=12.0, max_reps=1500):   # about 20 core-seconds on 16 threads
     threads = min(os.cpu_count() or 1, 16)
     reps, t0 = 0, time.perf_counter()
     while True:
