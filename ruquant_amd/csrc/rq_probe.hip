@@ -1,0 +1,196 @@
+// Machine-peak probes for gfx950, launched through rq_w4a4_probe() and timed by the caller (bench.py captures a
+// batch of launches in a HIP graph and brackets it with events, exactly as it times the operator).
+//
+// They answer the questions the operator's kernels are judged against:
+//   * how fast a plain kernel streams a given number of bytes from HBM (the ceiling of the GEMV),
+//   * how fast the matrix pipe runs v_mfma_i32_16x16x64_i8 alone (the ceiling of the GEMM),
+//   * whether vector-ALU instructions overlap with MFMAs: in one wavefront, and between two wavefronts that share
+//     a SIMD, one issuing only MFMAs and the other only VALU (the per-group integer fold of the W4A4 format is VALU
+//     work beside every MFMA),
+//   * what an (almost) empty kernel costs per launch inside a graph (the floor of a two-kernel decode op).
+// The method follows the reference's rig/membench/stream_bench.hip and rig/bench_valu.cu: dependent chains per
+// register so that nothing can be optimized away, independent chains across registers so that issue, not latency,
+// is measured.
+#include "rq_common.h"
+
+namespace rq {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(256) probe_empty_kernel(int *sink) {
+    if (sink == nullptr && threadIdx.x == 12345) __builtin_trap();
+}
+
+// Streaming read: workgroup b takes chunks b, b + grid, ... of U KiB-per-wavefront loads (U x 4 KiB per workgroup);
+// all U loads of a thread are in flight before the first is consumed. Loads are non-temporal, like the GEMV's.
+template <int U>
+__global__ void __launch_bounds__(256) probe_stream_kernel(const v4u *__restrict__ p, int64_t chunks, int *sink) {
+    unsigned acc = 0;
+    for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+        const v4u *q = p + (c * U) * 256 + threadIdx.x;
+        v4u v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(q + u * 256);
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    if (acc == 0x9e3779b9u) sink[0] = 1;   // the probe buffer holds small integers: never true
+}
+
+#define RQ_VALU8(OP)                                                                                   \
+    asm volatile(OP " %0, %8, %0\n\t" OP " %1, %8, %1\n\t" OP " %2, %8, %2\n\t" OP " %3, %8, %3\n\t"   \
+                 OP " %4, %8, %4\n\t" OP " %5, %8, %5\n\t" OP " %6, %8, %6\n\t" OP " %7, %8, %7"       \
+                 : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3), "+v"(x4), "+v"(x5), "+v"(x6), "+v"(x7)      \
+                 : "v"(y))
+
+// 16 MFMAs on four independent accumulators
+#define RQ_MFMA16()                                                             \
+    _Pragma("unroll") for (int r = 0; r < 16; ++r)                              \
+        c[r & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c[r & 3], 0, 0, 0)
+
+// role of a wavefront: bit 0 = issues MFMAs, bit 1 = issues VALU. Wavefronts w and w + 4 of a workgroup share a SIMD
+// (the hardware deals a workgroup's wavefronts to the four SIMDs in turn; `simd_of` records where each one ran so
+// that the caller can check it).
+//   SAME  = true : every wavefront interleaves 1 MFMA with NV VALU instructions (roles ignored)
+//   SAME  = false: wavefronts 0..3 take role_lo, wavefronts 4..7 role_hi
+// OPK: 0 = v_add_u32, 1 = v_ashrrev_i32, 2 = v_mul_i32_i24
+template <bool SAME, int NV, int OPK>
+__global__ void __launch_bounds__(512) probe_mix_kernel(int mfma_iters, int valu_iters, int role_lo, int role_hi,
+                                                        int *sink, int *simd_of) {
+    v4i a = { (int) threadIdx.x, 1, 2, 3 }, b = { 4, 5, 6, (int) threadIdx.x };
+    v4i c[4] = {};
+    int x0 = threadIdx.x, x1 = 1, x2 = 2, x3 = 3, x4 = 4, x5 = 5, x6 = 6, x7 = 7, y = threadIdx.x * 3 + 1;
+    const int wave = threadIdx.x >> 6;
+    if (simd_of != nullptr && blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
+        // HW_REG_HW_ID (4), bits 5:4 = SIMD id
+        simd_of[wave] = (int) __builtin_amdgcn_s_getreg((2 - 1) << 11 | 4 << 6 | 4);
+    }
+    if (SAME) {
+        for (int it = 0; it < mfma_iters; ++it) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                c[r & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c[r & 3], 0, 0, 0);
+                if (NV >= 8) {
+                    if (OPK == 0) RQ_VALU8("v_add_u32");
+                    if (OPK == 1) RQ_VALU8("v_ashrrev_i32");
+                    if (OPK == 2) RQ_VALU8("v_mul_i32_i24");
+                }
+                if (NV >= 16) {
+                    if (OPK == 0) RQ_VALU8("v_add_u32");
+                    if (OPK == 1) RQ_VALU8("v_ashrrev_i32");
+                    if (OPK == 2) RQ_VALU8("v_mul_i32_i24");
+                }
+            }
+        }
+    } else {
+        const int role = wave < 4 ? role_lo : role_hi;
+        if (role & 1) {
+            for (int it = 0; it < mfma_iters; ++it) {
+                RQ_MFMA16();
+            }
+        }
+        if (role & 2) {
+            for (int it = 0; it < valu_iters; ++it) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    if (OPK == 0) RQ_VALU8("v_add_u32");
+                    if (OPK == 1) RQ_VALU8("v_ashrrev_i32");
+                    if (OPK == 2) RQ_VALU8("v_mul_i32_i24");
+                }
+            }
+        }
+    }
+    if (c[0][0] + c[1][1] + c[2][2] + c[3][3] + x0 + x1 + x2 + x3 + x4 + x5 + x6 + x7 == 0x7fffffff) sink[0] = 1;
+}
+
+template <int OPK>
+hipError_t launch_mix(int sub, int grid, int block, int mi, int vi, int *sink, int *simd_of, hipStream_t s) {
+    switch (sub) {
+        case 0:   // all wavefronts: MFMA only
+            hipLaunchKernelGGL((probe_mix_kernel<false, 0, OPK>), dim3(grid), dim3(block), 0, s, mi, vi, 1, 1, sink, simd_of);
+            break;
+        case 1:   // all wavefronts: VALU only
+            hipLaunchKernelGGL((probe_mix_kernel<false, 0, OPK>), dim3(grid), dim3(block), 0, s, mi, vi, 2, 2, sink, simd_of);
+            break;
+        case 2:   // wavefronts 0..3 MFMA, 4..7 VALU: one of each on every SIMD
+            hipLaunchKernelGGL((probe_mix_kernel<false, 0, OPK>), dim3(grid), dim3(block), 0, s, mi, vi, 1, 2, sink, simd_of);
+            break;
+        case 3:   // wavefronts 0..3 MFMA, 4..7 idle
+            hipLaunchKernelGGL((probe_mix_kernel<false, 0, OPK>), dim3(grid), dim3(block), 0, s, mi, vi, 1, 0, sink, simd_of);
+            break;
+        case 4:   // wavefronts 0..3 idle, 4..7 VALU
+            hipLaunchKernelGGL((probe_mix_kernel<false, 0, OPK>), dim3(grid), dim3(block), 0, s, mi, vi, 0, 2, sink, simd_of);
+            break;
+        case 5:   // one wavefront: 1 MFMA + 8 VALU, interleaved
+            hipLaunchKernelGGL((probe_mix_kernel<true, 8, OPK>), dim3(grid), dim3(block), 0, s, mi, vi, 3, 3, sink, simd_of);
+            break;
+        case 6:   // one wavefront: 1 MFMA + 16 VALU, interleaved
+            hipLaunchKernelGGL((probe_mix_kernel<true, 16, OPK>), dim3(grid), dim3(block), 0, s, mi, vi, 3, 3, sink, simd_of);
+            break;
+        case 7:   // every wavefront: its MFMAs first, then its VALU work (no interleaving inside a wavefront)
+            hipLaunchKernelGGL((probe_mix_kernel<false, 0, OPK>), dim3(grid), dim3(block), 0, s, mi, vi, 3, 3, sink, simd_of);
+            break;
+        default:
+            return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace
+}  // namespace rq
+
+using namespace rq;
+
+extern "C" int rq_w4a4_probe(int kind, int64_t a0, int64_t a1, int64_t a2, int64_t a3, void *buf, size_t bytes,
+                             rq_stream_t stream) {
+    hipStream_t s = (hipStream_t) stream;
+    if (!buf || bytes < 4096 || (reinterpret_cast<uintptr_t>(buf) & 255) != 0) return RQ_E_ARGUMENT;
+    int *sink = reinterpret_cast<int *>(buf);   // never written (the conditions above are never true)
+    switch (kind) {
+        case RQ_PROBE_EMPTY: {
+            if (a0 < 1 || a0 > 65536) return RQ_E_ARGUMENT;
+            hipLaunchKernelGGL(probe_empty_kernel, dim3((unsigned) a0), dim3(256), 0, s, sink);
+            return (int) hipGetLastError();
+        }
+        case RQ_PROBE_STREAM: {
+            // a0 = bytes to read, a1 = 16-byte loads in flight per thread, a2 = workgroups (0: one per chunk)
+            const int64_t U = a1;
+            if (U != 4 && U != 5 && U != 8 && U != 10 && U != 16 && U != 20) return RQ_E_ARGUMENT;
+            const int64_t chunk = U * 4096;
+            if (a0 < chunk || a0 % chunk != 0 || (size_t) a0 > bytes) return RQ_E_ARGUMENT;
+            const int64_t chunks = a0 / chunk;
+            const int64_t grid = a2 > 0 ? a2 : chunks;
+            if (grid > (1 << 24)) return RQ_E_ARGUMENT;
+            const v4u *p = reinterpret_cast<const v4u *>(buf);
+            int *snk = sink;
+            switch (U) {
+                case 4:  hipLaunchKernelGGL(probe_stream_kernel<4>, dim3((unsigned) grid), dim3(256), 0, s, p, chunks, snk); break;
+                case 5:  hipLaunchKernelGGL(probe_stream_kernel<5>, dim3((unsigned) grid), dim3(256), 0, s, p, chunks, snk); break;
+                case 8:  hipLaunchKernelGGL(probe_stream_kernel<8>, dim3((unsigned) grid), dim3(256), 0, s, p, chunks, snk); break;
+                case 10: hipLaunchKernelGGL(probe_stream_kernel<10>, dim3((unsigned) grid), dim3(256), 0, s, p, chunks, snk); break;
+                case 16: hipLaunchKernelGGL(probe_stream_kernel<16>, dim3((unsigned) grid), dim3(256), 0, s, p, chunks, snk); break;
+                default: hipLaunchKernelGGL(probe_stream_kernel<20>, dim3((unsigned) grid), dim3(256), 0, s, p, chunks, snk); break;
+            }
+            return (int) hipGetLastError();
+        }
+        case RQ_PROBE_MIX: {
+            // a0 = sub-kind | VALU instruction << 8, a1 = workgroups, a2 = MFMA iterations (16 MFMAs each),
+            // a3 = VALU iterations (128 instructions each). Workgroups are 512 threads (two wavefronts per SIMD), or
+            // 256 threads for the one-wavefront-per-SIMD interleaved forms (sub-kinds 5 and 6 with bit 16 set).
+            const int sub = (int) (a0 & 0xFF), opk = (int) ((a0 >> 8) & 0xFF);
+            const int block = (a0 >> 16) & 1 ? 256 : 512;
+            if (a1 < 1 || a1 > 65536 || a2 < 0 || a3 < 0 || a2 > (1 << 24) || a3 > (1 << 24)) return RQ_E_ARGUMENT;
+            int *simd_of = bytes >= 8192 ? sink + 1024 : nullptr;   // 8 ints at byte 4096
+            switch (opk) {
+                case 0: return (int) launch_mix<0>(sub, (int) a1, block, (int) a2, (int) a3, sink, simd_of, s);
+                case 1: return (int) launch_mix<1>(sub, (int) a1, block, (int) a2, (int) a3, sink, simd_of, s);
+                case 2: return (int) launch_mix<2>(sub, (int) a1, block, (int) a2, (int) a3, sink, simd_of, s);
+                default: return RQ_E_ARGUMENT;
+            }
+        }
+        default:
+            return RQ_E_ARGUMENT;
+    }
+}

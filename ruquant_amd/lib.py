@@ -65,6 +65,8 @@ PROTOTYPES = {
                                                 ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "rq_w4a4_dequantize": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
                                           ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
+    "rq_w4a4_probe": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                     ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "rq_w4a4_quantize_act": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
                                             ctypes.c_int64, ctypes.c_float, ctypes.c_int64, ctypes.c_void_p,
                                             ctypes.c_void_p]),
