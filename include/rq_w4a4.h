@@ -38,6 +38,7 @@ extern "C" {
 #define RQ_E_UNSUPPORTED  (-1)  /* shape/type the op does not take (the reference says so via supports_op) */
 #define RQ_E_WORKSPACE    (-2)  /* workspace or prepared buffer too small or misaligned */
 #define RQ_E_ARGUMENT     (-3)  /* null pointer, bad clip, bad rotation length */
+#define RQ_E_LIMIT        (-4)  /* rq_w4a4_mul_mat_static: the problem needs more than RQ_STATIC_SCRATCH_BYTES */
 
 typedef void *rq_stream_t;
 
@@ -99,6 +100,21 @@ int rq_w4a4_mul_mat(int type, const void *prepared_dev, int64_t K, int64_t N,
                     float *y_dev, int64_t ldy,
                     float clip, int64_t n_rot,
                     void *workspace_dev, size_t workspace_bytes, rq_stream_t stream);
+
+/* rq_w4a4_mul_mat for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): no counterpart in the reference, which takes its scratch from the backend pool.
+ * Same arguments and results as rq_w4a4_mul_mat without the workspace: the scratch is a 16 MiB array inside the
+ * library's code object (one copy per GPU, held until the process ends). Allocates nothing and frees nothing.
+ * Returns RQ_E_LIMIT when rq_w4a4_workspace_bytes(type, K, N, M) exceeds RQ_STATIC_SCRATCH_BYTES (decode and
+ * verify batches fit: K = 5120, N = 17408 up to 128 tokens; K = 32768, N = 65536 at 8). All calls on one GPU share
+ * the array: calls that overlap in time on one GPU (two streams, two threads) race; serialize them or give the
+ * others rq_w4a4_mul_mat with workspaces of their own. rq_w4a4_prepare on the same GPU must have run before (it
+ * resolves the array's device address, which must not happen under capture). */
+#define RQ_STATIC_SCRATCH_BYTES (16 << 20)
+int rq_w4a4_mul_mat_static(int type, const void *prepared_dev, int64_t K, int64_t N,
+                           const float *x_dev, int64_t ldx, int64_t M,
+                           float *y_dev, int64_t ldy,
+                           float clip, int64_t n_rot, rq_stream_t stream);
 
 /* Measurement aid with no counterpart in the reference: rq_w4a4_mul_mat split into its two stages so that the
  * product kernel can be timed alone. stages = 1: activation transform only (Hadamard + quantizer, also clears the

@@ -6,6 +6,13 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
+
+// Workspace of rq_w4a4_mul_mat_static: one array per GPU, part of the code object, so that callers which cannot
+// allocate device memory (HIP graph capture, serving loops) need none. In host code the array's name is only a handle
+// for hipGetSymbolAddress; every use goes through the per-device address that static_scratch() keeps.
+static __device__ __align__(256) unsigned char scratch[RQ_STATIC_SCRATCH_BYTES];
+
 namespace rq {
 
 // same search as the reference's ggml_rq_hadamard_factor (reference patch lines 2419-2430): smallest p first
@@ -66,6 +73,33 @@ struct Env {
 const Env &env() {
     static const Env e;
     return e;
+}
+
+// Device address of `scratch` on the current device, resolved once per device (each GPU holds its own copy of the
+// array at its own address). Returns null with *err set when the runtime refuses.
+constexpr int kMaxDevices = 64;
+void *static_scratch(hipError_t *err) {
+    static std::mutex mu;
+    static void *ptr[kMaxDevices] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess && (dev < 0 || dev >= kMaxDevices)) e = hipErrorInvalidDevice;
+    if (e != hipSuccess) {
+        *err = e;
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            *err = e != hipSuccess ? e : hipErrorInvalidSymbol;
+            return nullptr;
+        }
+        ptr[dev] = p;
+    }
+    *err = hipSuccess;
+    return ptr[dev];
 }
 
 bool is_w_type(int type) { return type == RQ_TYPE_W4A4 || type == RQ_TYPE_W4A4H; }
@@ -319,6 +353,7 @@ int rq_w4a4_prepare(const void *w_blocks_dev, int64_t K, int64_t N, void *prepar
     // first use of a weight on this device: also the place for set-up that must not happen under graph capture
     hipError_t e = init_rotate_quant_kernels();
     if (e == hipSuccess) e = init_rotate_slab_kernels();
+    if (e == hipSuccess) static_scratch(&e);   // this device's address of the static workspace
     if (e != hipSuccess) return (int) e;
     return (int) launch_prepare(w_blocks_dev, L, reinterpret_cast<uint8_t *>(prepared_dev), (hipStream_t) stream);
 }
@@ -333,6 +368,17 @@ int rq_w4a4_mul_mat(int type, const void *prepared_dev, int64_t K, int64_t N, co
                     size_t workspace_bytes, rq_stream_t stream) {
     return run_products(type, 1, &prepared_dev, K, &N, x_dev, ldx, M, &y_dev, &ldy, clip, n_rot, workspace_dev,
                         workspace_bytes, (hipStream_t) stream);
+}
+
+int rq_w4a4_mul_mat_static(int type, const void *prepared_dev, int64_t K, int64_t N, const float *x_dev, int64_t ldx,
+                           int64_t M, float *y_dev, int64_t ldy, float clip, int64_t n_rot, rq_stream_t stream) {
+    if (!shape_ok(type, K, N, M)) return RQ_E_UNSUPPORTED;
+    if (workspace_layout(K, N, M < 1 ? 1 : M).bytes > (size_t) RQ_STATIC_SCRATCH_BYTES) return RQ_E_LIMIT;
+    hipError_t e = hipSuccess;
+    void *ws = static_scratch(&e);   // resolved by rq_w4a4_prepare on this device; here only looked up
+    if (!ws) return (int) e;
+    return run_products(type, 1, &prepared_dev, K, &N, x_dev, ldx, M, &y_dev, &ldy, clip, n_rot, ws,
+                        (size_t) RQ_STATIC_SCRATCH_BYTES, (hipStream_t) stream);
 }
 
 int rq_w4a4_mul_mat_stages(int type, const void *prepared_dev, int64_t K, int64_t N, const float *x_dev, int64_t ldx,
