@@ -8,11 +8,18 @@ stated on: W4A4H, K = 5120, N = 17408, M = 1, reported as GB/s of algorithmic by
 of the weight to exceed the 256 MB Infinity Cache, so the codes come from HBM.
 
 Prints one JSON line. Besides the contract fields it carries
-  roofline     : the product kernel alone (HIP events around back-to-back launches on the launch stream),
-  cpu_baseline : the CPU oracle (a bit-identical restatement of the ggml-cpu reference path) on the host cores,
-  extra        : the same measurements for the other benchmark shapes (M = 2048 prefill as TOPS against the dense
-                 int8 MFMA peak, the N = 5120 decode shapes, the K = 17408 down projection) and the seven matmuls of
-                 one transformer layer at 16 tokens and at one token, run in the layer's dataflow.
+  roofline       : the product kernel of the headline alone (HIP events around back-to-back launches on the launch
+                   stream), against the HBM peak,
+  roofline_m2048 : the tiled MFMA GEMM alone at M = 2048 (K = 5120, N = 17408), against the dense int8 MFMA peak: the
+                   second half of the metric,
+  cpu_baseline   : the CPU oracle (a bit-identical restatement of the ggml-cpu reference path) on the host cores,
+  extra          : the same measurements for the other benchmark shapes (the N = 5120 decode shapes, the K = 17408 down
+                   projection, the reference's perf-mode shape 6144 x 5120), the seven matmuls of one transformer
+                   layer at 16 tokens and at one token, run in the layer's dataflow, and `peaks`: what this machine
+                   delivers to plain probe kernels in the same run (a streaming read of the headline's byte count, a
+                   pure v_mfma_i32_16x16x64_i8 loop, vector-ALU instructions beside MFMAs in one wavefront and in two
+                   wavefronts that share a SIMD, an empty launch).
+Every time is the median over batches of back-to-back launches captured in one HIP graph.
 """
 import argparse
 import json
@@ -25,10 +32,21 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
-# HBM bytes per launch of the headline product kernel: rocprofv3 FETCH_SIZE 21,923.0 KiB / 0.500 (scale from a plain
-# copy of known size) + WRITE_SIZE 748.0 KiB / 1.000, from the runs summarized in profiles/gemv_m1_k5120_n17408.md
-HEADLINE_TRAFFIC_BYTES = int((21923.0 / 0.500 + 748.0) * 1024)
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA
+# HBM bytes per launch of the headline's dominant kernel come from the committed rocprofv3 counter summary (FETCH_SIZE
+# and WRITE_SIZE passes, each scaled by a plain copy of known size): the line "traffic_bytes_per_launch: <n>" in it
+HEADLINE_PROFILE = os.path.join(ROOT, "profiles", "gemv_m1_k5120_n17408.md")
+
+
+def profiled_traffic_bytes(path=HEADLINE_PROFILE):
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return int(line.split(":")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def algorithmic_bytes(K, N, M):
@@ -199,8 +217,18 @@ class Layer:
                 "layer_us_seven_separate_calls": round(plain_ms * 1e3, 2)}
 
 
+def host_cores():
+    """(logical CPUs the machine reports, CPUs this process may run on)."""
+    n = os.cpu_count() or 1
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        usable = n
+    return n, usable
+
+
 def cpu_baseline(oracle, prob, budget_s=12.0, max_reps=1500):   # about 20 core-seconds on 16 threads
-    threads = min(os.cpu_count() or 1, 16)
+    threads = min(host_cores()[1], 16)
     reps, t0 = 0, time.perf_counter()
     while True:
         oracle.mul_mat(prob.type, prob.blocks, prob.x_host, prob.clip, n_rot=prob.K, n_threads=threads)
@@ -212,7 +240,8 @@ def cpu_baseline(oracle, prob, budget_s=12.0, max_reps=1500):   # about 20 core-
 
 
 def measure(prob, steps, warmup, bound):
-    op_ms, wall_ms = prob.timed(steps, warmup, 3)
+    _, wall_ms = prob.timed(steps, warmup, 3)
+    op_ms = prob.median_timed(steps, 2, 3)
     kern_ms = prob.median_timed(steps, warmup, 2)
     act_ms = prob.median_timed(steps, warmup, 1)
     K, N, M = prob.K, prob.N, prob.M
@@ -231,6 +260,98 @@ def measure(prob, steps, warmup, bound):
     return out, op_ms, kern_ms
 
 
+def machine_peaks(torch, rq, code_bytes, batches=5):
+    """What plain probe kernels of the library reach on this machine, measured like the operator (graph-captured
+    batches between events): see rq_w4a4_probe in include/rq_w4a4.h."""
+    import ctypes
+    L = rq.load_library()
+    dev = "cuda:0"
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+
+    def timed(fn, n):
+        for i in range(2):
+            fn(i)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(n):
+                fn(i)
+        g.replay()
+        torch.cuda.synchronize()
+        vals = []
+        for _ in range(batches):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            vals.append(e0.elapsed_time(e1) / n * 1e3)
+        return sorted(vals)[len(vals) // 2]
+
+    def probe(buf, kind, a0, a1=0, a2=0, a3=0, off=0, nbytes=None):
+        rc = L.rq_w4a4_probe(kind, a0, a1, a2, a3, buf.data_ptr() + off, buf.numel() - off if nbytes is None else nbytes,
+                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        if rc != 0:
+            raise RuntimeError("rq_w4a4_probe(%d) failed: %d" % (kind, rc))
+
+    out = {"compute_units": cus}
+    small = torch.zeros(1 << 16, dtype=torch.uint8, device=dev)
+    out["empty_launch_us"] = round(timed(lambda i: probe(small, 0, 1088), 50), 3)
+
+    # streaming read of the headline's code bytes, rotating over more than the memory-side cache holds
+    copies = max(2, -(-(320 << 20) // code_bytes))
+    big = torch.ones(copies * code_bytes // 4, dtype=torch.int32, device=dev).view(torch.uint8)
+    best = None
+    for loads in (5, 10):
+        if code_bytes % (loads * 4096):
+            continue
+        us = timed(lambda i: probe(big, 1, code_bytes, loads, 0, off=(i % copies) * code_bytes, nbytes=code_bytes), 3 * copies)
+        if best is None or us < best[0]:
+            best = (us, loads)
+    if best:
+        out["stream_read"] = {"bytes": code_bytes, "us": round(best[0], 3), "gbs": round(code_bytes / best[0] / 1e3, 1),
+                              "loads_in_flight_per_thread": best[1], "source": "HBM (%d rotating buffers)" % copies}
+        us = timed(lambda i: probe(big, 1, code_bytes, best[1], 0, off=0, nbytes=code_bytes), 24)
+        out["stream_read_cache_resident"] = {"bytes": code_bytes, "us": round(us, 3), "gbs": round(code_bytes / us / 1e3, 1)}
+        nb = copies * code_bytes // (best[1] * 4096) * (best[1] * 4096)
+        us = timed(lambda i: probe(big, 1, nb, best[1], 0, off=0, nbytes=nb), 4)
+        out["stream_read_large"] = {"bytes": nb, "us": round(us, 3), "gbs": round(nb / us / 1e3, 1)}
+    del big
+
+    # matrix pipe and vector ALU: workgroups of 8 wavefronts (two per SIMD), one workgroup per compute unit
+    ops_per_mfma = 16 * 16 * 64 * 2
+    mi, vi = 2000, 1000
+
+    def mix(sub, valu_op=0, one_wave_per_simd=False, m=mi, v=vi):
+        return timed(lambda i: probe(small, 2, sub | valu_op << 8 | (1 << 16 if one_wave_per_simd else 0), cus, m, v), 4)
+
+    simds = cus * 4
+    t = mix(3)
+    out["mfma_i8_16x16x64_tops_one_wavefront_per_simd"] = round(cus * 4 * mi * 16 * ops_per_mfma / t / 1e6, 1)
+    out["mfma_ns_per_instruction_per_simd"] = round(t * 1e3 / (mi * 16), 3)
+    t = mix(0)
+    out["mfma_i8_16x16x64_tops_two_wavefronts_per_simd"] = round(cus * 8 * mi * 16 * ops_per_mfma / t / 1e6, 1)
+    for op, name in ((0, "v_add_u32"), (1, "v_ashrrev_i32"), (2, "v_mul_i32_i24")):
+        t1, t2 = mix(4, op), mix(1, op)
+        out["valu_ns_per_instruction_per_simd_%s" % name] = {"one_wavefront": round(t1 * 1e3 / (vi * 128), 3),
+                                                             "two_wavefronts": round(t2 * 1e3 / (2 * vi * 128), 3)}
+    # one wavefront per SIMD issues only MFMAs, a second one on the same SIMD only v_add_u32
+    t_m, t_v, t_both = mix(3), mix(4), mix(2)
+    out["mfma_wavefront_beside_valu_wavefront_us"] = {"mfma_alone": round(t_m, 1), "valu_alone": round(t_v, 1),
+                                                      "together": round(t_both, 1), "sum": round(t_m + t_v, 1)}
+    # two wavefronts per SIMD of each kind (two workgroups per compute unit): the vector ALU at its full issue rate
+    def mix2(sub):
+        return timed(lambda i: probe(small, 2, sub, 2 * cus, mi, vi), 4)
+    t_m, t_v, t_both = mix2(3), mix2(4), mix2(2)
+    out["two_mfma_wavefronts_beside_two_valu_wavefronts_us"] = {"mfma_alone": round(t_m, 1), "valu_alone": round(t_v, 1),
+                                                                "together": round(t_both, 1), "sum": round(t_m + t_v, 1)}
+    # one wavefront interleaving 1 MFMA with 8 independent v_add_u32 (two such wavefronts per SIMD)
+    t = mix(5, 0, False, mi // 4, 0)
+    out["same_wavefront_1_mfma_8_valu_ns_per_mfma_per_simd"] = round(t * 1e3 / (2 * (mi // 4) * 16), 3)
+    out["same_wavefront_1_mfma_8_valu_tops"] = round(cus * 8 * (mi // 4) * 16 * ops_per_mfma / t / 1e6, 1)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -241,6 +362,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy 10 times (scale for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--shapes", default="", help="comma-separated names of the extra shapes to run (default: all)")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the machine-peak probes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this operator is measured on one GPU; --gpus %d is not a configuration of this build "
@@ -273,11 +395,18 @@ def main():
         from oracle import rq_oracle
         parity = head.check(rq_oracle)
         sec, reps, threads = cpu_baseline(rq_oracle, head)
-        cpu = {"value": round(b / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+        nproc, usable = host_cores()
+        cpu = {"value": round(b / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "nproc": nproc,
+               "cpus_usable": usable, "kind": "port",
                "sample": "%d whole-op passes of the same K=%d N=%d M=%d problem (%.2f ms each), CPU oracle, "
                          "two-phase threading" % (reps, K, N, M, sec * 1e3)}
 
     extra = {"headline": res}
+    if not args.no_peaks:
+        head = None
+        torch.cuda.empty_cache()
+        extra["peaks"] = machine_peaks(torch, rq, N * K // 2)
+    roofline_m2048 = None
     if not args.no_extra:
         shapes = [
             ("decode_k5120_n5120_m1", 5120, 5120, 1, "outlier_channels", 0.9, "hbm"),
@@ -288,6 +417,11 @@ def main():
             ("prefill_k5120_n17408_m512", 5120, 17408, 512, "student_t4", 0.85, "mfma"),
             ("prefill_k5120_n17408_m2048", 5120, 17408, 2048, "student_t4", 0.85, "mfma"),
             ("down_k17408_n5120_m2048", 17408, 5120, 2048, "relu2", 1.0, "mfma"),
+            # the reference's perf-mode shape (test-backend-ops perf, patch lines 3067-3074)
+            ("perf_k5120_n6144_m1", 5120, 6144, 1, "normal", 1.0, "hbm"),
+            ("perf_k5120_n6144_m8", 5120, 6144, 8, "normal", 1.0, "hbm"),
+            ("perf_k5120_n6144_m16", 5120, 6144, 16, "normal", 1.0, "hbm"),
+            ("perf_k5120_n6144_m512", 5120, 6144, 512, "normal", 1.0, "mfma"),
         ]
         want = [w for w in args.shapes.split(",") if w]
         for name, k, n, m, kind, clip, bound in shapes:
@@ -297,8 +431,16 @@ def main():
             torch.cuda.empty_cache()
             head = None
             head = Problem(k, n, m, kind, clip, seed=3)
-            steps = args.steps if m <= 64 else max(5, args.steps // 10)
-            extra[name], _, _ = measure(head, steps, min(args.warmup, steps), bound)
+            steps = args.steps if m <= 64 else max(20, args.steps // 10)
+            extra[name], _, kms = measure(head, steps, min(args.warmup, steps), bound)
+            if name == "prefill_k5120_n17408_m2048":
+                ops = 2.0 * m * n * k
+                roofline_m2048 = {"bound": "mfma", "achieved": round(ops / kms / 1e9, 1), "peak": INT8_PEAK_TOPS,
+                                  "unit": "TOP/s", "frac": round(ops / kms / 1e9 / INT8_PEAK_TOPS, 4), "traffic": None,
+                                  "kernel": "rq_gemm_kernel (wide + narrow tiles of one launch)",
+                                  "kernel_us": round(kms * 1e3, 3), "workload": "W4A4H K=5120 N=17408 M=2048",
+                                  "op_us": extra[name]["op_us"], "op_tops": extra[name]["op_tops"],
+                                  "op_frac": extra[name]["op_frac_of_int8_peak"]}
 
         for name, m in (("layer_m16", 16), ("layer_m1", 1)):
             if not want or name in want:
@@ -317,8 +459,9 @@ def main():
                                "outlier-channel activations), whole op, weights rotated over >256 MB",
                    "algorithmic_bytes": b},
         "roofline": {"bound": "hbm", "achieved": round(b / kern_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(b / kern_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": HEADLINE_TRAFFIC_BYTES,
+                     "frac": round(b / kern_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": profiled_traffic_bytes(),
                      "kernel": "rq_gemv_kernel<1, 4, 1>", "kernel_us": round(kern_ms * 1e3, 3)},
+        "roofline_m2048": roofline_m2048,
         "cpu_baseline": cpu,
         "parity_vs_oracle": parity,
         "extra": extra,

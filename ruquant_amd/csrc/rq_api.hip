@@ -49,6 +49,7 @@ struct Env {
     int   gemm_min;  // smallest token count that takes the tiled MFMA GEMM
     int   gemv_max;  // largest token count that takes the GEMV; between the two: the skinny MFMA kernel
     int   skinny_single;  // skinny path: single-plane activations (RQ_SKINNY_SINGLE=0 switches back to two digits)
+    int   decode_fused;   // one token: the single-launch kernel (RQ_DECODE_FUSED=0: rotation kernel + GEMV)
     Env() {
         const char *e = getenv("RQ_ACT_CLIP");
         const char *eh = getenv("RQ_ACT_CLIP_H");
@@ -67,6 +68,8 @@ struct Env {
         if (gemv_max > kGemvMaxTokens) gemv_max = kGemvMaxTokens;
         const char *ss = getenv("RQ_SKINNY_SINGLE");
         skinny_single = ss ? atoi(ss) != 0 : 1;
+        const char *df = getenv("RQ_DECODE_FUSED");
+        decode_fused = df ? atoi(df) != 0 : 1;
     }
 };
 
@@ -100,6 +103,21 @@ void *static_scratch(hipError_t *err) {
     }
     *err = hipSuccess;
     return ptr[dev];
+}
+
+// Compute units of the current device, read once per device (first use of a weight; a later call only looks it up).
+int device_compute_units() {
+    static std::mutex mu;
+    static int cus[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+    std::lock_guard<std::mutex> lock(mu);
+    if (cus[dev] == 0) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) return 0;
+        cus[dev] = v;
+    }
+    return cus[dev];
 }
 
 bool is_w_type(int type) { return type == RQ_TYPE_W4A4 || type == RQ_TYPE_W4A4H; }
@@ -167,6 +185,29 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     // that only the narrow-tile MFMA kernel does (44 us from 4 to 64 tokens), so every larger token count takes it
     // (a format variant, not a tuned path).
     const int G = env().act_group;
+    if (M == 1 && env().decode_fused && decode_takes((int) K, type == RQ_TYPE_W4A4H, p, m, G)) {
+        // one token: rotation, quantizer, product and epilogue in one launch, all weights of a fused call included
+        if (!(stages & 2)) return 0;
+        DecodeArgs d;
+        memset(&d, 0, sizeof d);
+        d.w.n = n;
+        for (int i = 0; i < n; ++i) {
+            d.w.prepared[i] = reinterpret_cast<const uint8_t *>(prepared[i]);
+            d.w.L[i] = prepared_layout(K, N[i]);
+            d.w.y[i] = y[i];
+            d.w.ldy[i] = ldy[i];
+        }
+        d.x = x;
+        d.K = (int) K;
+        d.rotate = type == RQ_TYPE_W4A4H;
+        d.n_rot = (int) (d.rotate ? n_rot : K);
+        d.p = p;
+        d.m = m;
+        d.scale = 1.0f / sqrtf((float) d.n_rot);
+        d.clip = clip;
+        d.compute_units = device_compute_units();
+        return (int) launch_decode(d, stream);
+    }
     const Path path = G != 64 ? (M <= kGemvWideTokens ? kPathGemv : kPathGemm) : path_of(M);
     const bool gemm = path != kPathGemv;   // the int8 digit planes feed both MFMA kernels
     RotQuantArgs q;
@@ -353,7 +394,9 @@ int rq_w4a4_prepare(const void *w_blocks_dev, int64_t K, int64_t N, void *prepar
     // first use of a weight on this device: also the place for set-up that must not happen under graph capture
     hipError_t e = init_rotate_quant_kernels();
     if (e == hipSuccess) e = init_rotate_slab_kernels();
+    if (e == hipSuccess) e = init_decode_kernels();
     if (e == hipSuccess) static_scratch(&e);   // this device's address of the static workspace
+    device_compute_units();
     if (e != hipSuccess) return (int) e;
     return (int) launch_prepare(w_blocks_dev, L, reinterpret_cast<uint8_t *>(prepared_dev), (hipStream_t) stream);
 }

@@ -245,6 +245,20 @@ struct SkinnyPlan {
 };
 SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz);
 
+// One token, one launch (rq_decode.hip): every workgroup rotates and quantizes the token for itself behind its share of
+// the weight stream; rows are dealt in quads, whole K per workgroup, so no sums cross workgroups.
+constexpr int kDecodeCells = 512;   // most rows of one workgroup: its LDS cells (one per row)
+struct DecodeArgs {
+    FusedWeights    w;
+    const float    *x;        // the token's row
+    int             K, rotate, n_rot, p, m;
+    float           scale, clip;
+    int             compute_units;   // of the device (0: unknown)
+};
+hipError_t launch_decode(const DecodeArgs &a, hipStream_t stream);
+hipError_t init_decode_kernels();
+bool decode_takes(int K, int rotate, int p, int m, int act_group);
+
 hipError_t launch_prepare(const void *blocks, const PreparedLayout &L, uint8_t *prepared, hipStream_t stream);
 
 bool hadamard_factor(int64_t n, int &p, int &m);

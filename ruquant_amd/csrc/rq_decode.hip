@@ -1,0 +1,592 @@
+// One-token W4A4 / W4A4H MUL_MAT in ONE launch: online Hadamard, activation quantizer, int4 x int4 product and the
+// fp32 epilogue (kernels 1-4 of the decode path) with no second kernel, no split-K cells and no atomics in memory.
+//
+// Why one launch: a dependent launch costs about 1.8 us on this part even inside a HIP graph, and the rotation of a
+// single row is a chain of short latency-bound phases that cannot fill the chip. Here every workgroup repeats the
+// (cheap) rotation + quantization of the token for itself, hidden behind its own share of the weight stream:
+//
+//   * wavefronts 8..15 ("stream") put ALL of the workgroup's weight bytes in flight into registers right away
+//     (about 170 KiB per compute unit for a 44 MB weight; a wavefront that has queued loads stalls at issue once the
+//     memory queue is full, which is why these wavefronts do nothing else), then wait at the workgroup's barriers;
+//   * wavefronts 0..7 ("rotate") load the row, run the Sylvester butterflies and the Paley stage in LDS with the
+//     reference's order of additions (ggml_rq_hadamard, reference patch lines 2450-2485), reduce the clipped group
+//     ranges, derive the token unit, the group multipliers and zero points and the 4-bit codes
+//     (rq_quantize_row_a, lines 2639-2679) into LDS;
+//   * the stream wavefronts then fold group by group (ggml_vec_dot_w4a4_a4, lines 148-177) as their loads arrive,
+//     add the exact int32 terms into per-row cells in LDS, and the epilogue writes y = ((float(total) * 16) * u) * s_w.
+//
+// Work is dealt in whole rows (never along K, so no reduction between workgroups exists): the rows of the launch are
+// cut into quads, workgroup s takes quads [s Q / G, (s + 1) Q / G), and G is the number of compute units, so every
+// compute unit streams the same number of bytes to within one quad. A stream wavefront reads the prepared layout as
+// items of 8 rows x 4 groups: lane = (row of the octet, half of the group, group of the item), one 16-byte load per
+// lane, eight full 128-byte lines per wavefront load. An octet that two workgroups share is read by both (its lines
+// hold both quads); the slot order puts such neighbours on one XCD, where the second read is an L2 hit.
+#include "rq_hadamard.h"
+
+#pragma clang fp contract(off)
+
+#ifdef RQ_DECODE_TIMING
+__device__ unsigned long long rq_decode_stamps[64];
+#define RQ_STAMP(i) do { if (blockIdx.x == 0 && (threadIdx.x == 0 || threadIdx.x == 512)) rq_decode_stamps[(i) + (threadIdx.x ? 32 : 0)] = __builtin_readcyclecounter(); } while (0)
+extern "C" int rq_w4a4_decode_stamps(unsigned long long *out) {
+    return (int) hipMemcpyFromSymbol(out, HIP_SYMBOL(rq_decode_stamps), sizeof(rq_decode_stamps));
+}
+#else
+#define RQ_STAMP(i) do { } while (0)
+#endif
+
+namespace rq {
+
+namespace {
+
+using namespace had;
+
+constexpr int kRotWaves = 8;
+constexpr int kStrWaves = 8;
+constexpr int kRotThreads = kRotWaves * 64;
+constexpr int kDecThreads = (kRotWaves + kStrWaves) * 64;
+
+struct DecodeKernelArgs {
+    WeightSet    ws;        // up to three weights of one K; first[] counts panels
+    const float *x;         // the token's row of K floats
+    int          K, rotate, n_rot, m;
+    float        scale, clip;
+    int          main_panels;       // whole panels per workgroup: panels s, s + G, ... (G = workgroups)
+    int          tail_panel0;       // first panel of the remainder, which is dealt in quads of rows
+    int          q_base, q_extra;   // remainder quads per workgroup: q_base, the first q_extra slots one more
+    int          n_pass;            // Sylvester passes through LDS after the register pass
+    int          inv_nblk;          // floor(2^22 / nblk) + 1, nblk = K / 256: i / nblk = (i * inv_nblk) >> 22 for every item index
+};
+
+__device__ __forceinline__ int dot8(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot8((int) a, (int) b, c, false);
+}
+
+__device__ __forceinline__ int align4(int v) { return (v + 3) & ~3; }
+
+// Barrier among the rotate wavefronts only, through a counter in LDS that only grows: a wavefront adds one when its
+// LDS writes of the phase are done and waits until all kRotWaves have (`target` = kRotWaves x phases so far). The
+// hardware barrier would also wait for the stream wavefronts, which sit blocked in the issue of their loads for
+// microseconds (the memory queue is full): the phases of the rotation must not wait for that.
+// (The counter is read through an LDS-typed pointer: a generic one makes the poll a FLAT load, which queues behind
+// the weight stream.)
+typedef __attribute__((address_space(3))) int lds_int;
+__device__ __forceinline__ void wait_count(const int *cnt, int target) {
+    const volatile lds_int *c = (const volatile lds_int *) cnt;
+    while (__builtin_amdgcn_readfirstlane(*c) < target) __builtin_amdgcn_s_sleep(1);
+    asm volatile("" ::: "memory");
+}
+__device__ __forceinline__ void rot_sync(int *cnt, int &target, int lane) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (lane == 0) atomicAdd(cnt, 1);
+    target += kRotWaves;
+    wait_count(cnt, target);
+}
+
+// LDS: [row][row (Paley output)][g_lo][g_hi][codes][mz][cells][wave maxima, unit]
+__host__ __device__ inline size_t decode_lds_bytes(int K, bool two_rows) {
+    const int Kp = ((K + (K >> 4) + 1) + 3) & ~3;
+    const int ng = K / kGroup;
+    return (size_t) ((two_rows ? 2 : 1) * Kp + 2 * ng + K / 8 + ng + kDecodeCells + 8 + kRotWaves + 4) * 4;
+}
+
+// MG: group-items (64 rows x one group: two loads) a stream wavefront has in flight per round of a whole panel;
+// MT: remainder items (8 rows x 4 groups: one load) per round. The first round of both is issued up front.
+template <int P, int MG, int MT>
+__global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKernelArgs a) {
+    extern __shared__ __align__(16) float smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    RQ_STAMP(0);
+    const int K = a.K, ng = K / kGroup;
+    const int Kp = align4(padi(K) + 1);
+    float *buf = smem;
+    float *alt = smem + Kp;
+    float *g_lo = smem + (P > 1 ? 2 : 1) * Kp;
+    float *g_hi = g_lo + ng;
+    uint32_t *s_act = reinterpret_cast<uint32_t *>(g_hi + ng);     // [K / 8] code words, tensor nibble order
+    int32_t *s_mz = reinterpret_cast<int32_t *>(s_act + K / 8);    // [ng] m | (8 - z) << 8
+    int32_t *red = s_mz + ng;                                      // cells: [whole panels][64 rows], [octets][8 rows], one spare
+    float *s_part = reinterpret_cast<float *>(red + kDecodeCells + 8);   // [kRotWaves] widest range per wavefront
+    float *s_unit = s_part + kRotWaves;
+    int *s_cnt = reinterpret_cast<int *>(s_unit + 1);   // phases the rotate wavefronts have finished, x kRotWaves
+
+    // ---- this workgroup's rows: whole panels s, s + G, ..., and a run of quads of the remainder panels. Remainder
+    // slots run over the XCDs so that slots t and t + 1 (which may share an octet) sit on one XCD: workgroups go to
+    // the eight XCDs round robin.
+    const int G = gridDim.x;
+    const int s_wg = blockIdx.x;
+    int slot = s_wg;
+    if ((G & 7) == 0) slot = (int) (blockIdx.x & 7) * (G >> 3) + (int) (blockIdx.x >> 3);
+    const int q0 = a.tail_panel0 * 16 + slot * a.q_base + (slot < a.q_extra ? slot : a.q_extra);
+    const int q1 = q0 + a.q_base + (slot < a.q_extra ? 1 : 0);
+    const int oct0 = q0 >> 1, n_oct = q1 > q0 ? ((q1 + 1) >> 1) - oct0 : 0;
+    const int nblk = ng >> 2;
+    const int main_cells = a.main_panels * kPanelRows;
+
+    // the epilogue's thread = one row of the workgroup; its row scale is requested before anything else
+    float pre_sw = 0.0f;
+    float *y_row = nullptr;
+    if (tid < main_cells + n_oct * 8) {
+        int panel, r;
+        bool mine = true;
+        if (tid < main_cells) {
+            panel = (tid >> 6) * G + s_wg;
+            r = tid & 63;
+        } else {
+            const int t = tid - main_cells;
+            const int o = oct0 + (t >> 3);
+            const int q = 2 * o + ((t & 7) >> 2);
+            panel = o >> 3;
+            r = (o & 7) * 8 + (t & 7);
+            mine = q >= q0 && q < q1;
+        }
+        const int wsel = (panel >= a.ws.first[1]) + (panel >= a.ws.first[2]);
+        const int wpanel = panel - (wsel == 0 ? 0 : wsel == 1 ? a.ws.first[1] : a.ws.first[2]);
+        const float *s_w = wsel == 0 ? a.ws.s_w[0] : wsel == 1 ? a.ws.s_w[1] : a.ws.s_w[2];
+        const int64_t N = wsel == 0 ? a.ws.N[0] : wsel == 1 ? a.ws.N[1] : a.ws.N[2];
+        float *y = wsel == 0 ? a.ws.y[0] : wsel == 1 ? a.ws.y[1] : a.ws.y[2];
+        const int64_t n = (int64_t) wpanel * kPanelRows + r;
+        if (mine && n < N) {
+            pre_sw = s_w[n];
+            y_row = y + n;
+        }
+        red[tid] = 0;
+    }
+    if (tid == 0) s_cnt[0] = 0;
+
+    if (wave >= kRotWaves) {
+        // =========================================================== the weight stream
+        const int sw = wave - kRotWaves;
+        const int r8 = lane & 7, h = (lane >> 3) & 1, g4 = lane >> 4;
+        const uint32_t lane_off = (uint32_t) (g4 * 2048 + h * 1024 + r8 * 16);
+        // flag words of the weights (bit 0: some weight multiplier differs from 1)
+        const int32_t f0 = __builtin_nontemporal_load(a.ws.flags[0]);
+        const int32_t f1 = __builtin_nontemporal_load(a.ws.flags[1]);
+        const int32_t f2 = __builtin_nontemporal_load(a.ws.flags[2]);
+
+        __builtin_amdgcn_s_barrier();   // the rotate wavefronts have the row
+        RQ_STAMP(1);
+
+        const bool anyk = ((f0 | f1 | f2) & 1) != 0;
+        const int n_items = n_oct * nblk;
+        const int codes_ready = kRotWaves * (1 + a.n_pass + (a.rotate ? 1 : 0) + 2);
+        typedef unsigned v4u __attribute__((ext_vector_type(4)));
+        bool waited = false;
+
+        // remainder item `i` of this workgroup -> address of its 1 KiB (8 rows x 4 groups x 2 halves)
+        // (items past the end read the first KiB of the remainder again: valid memory whatever this workgroup owns)
+        auto tail_address = [&](int i, bool valid) -> const uint8_t * {
+            const int ol = (int) (((uint32_t) i * (uint32_t) a.inv_nblk) >> 22);
+            const int bb = valid ? i - ol * nblk : 0;
+            const int o = valid ? oct0 + ol : a.tail_panel0 * 8;
+            const int panel = o >> 3;
+            const int wsel = (panel >= a.ws.first[1]) + (panel >= a.ws.first[2]);
+            const int wpanel = panel - (wsel == 0 ? 0 : wsel == 1 ? a.ws.first[1] : a.ws.first[2]);
+            const uint8_t *codes = wsel == 0 ? a.ws.codes[0] : wsel == 1 ? a.ws.codes[1] : a.ws.codes[2];
+            return codes + ((size_t) wpanel * ng + 4 * bb) * 2048 + (o & 7) * 128 + lane_off;
+        };
+        // the first round of remainder items goes out with the first round of the whole panels
+        v4u wt[MT > 0 ? MT : 1];
+        if constexpr (MT > 0) {
+#pragma unroll
+            for (int it = 0; it < MT; ++it) {
+                const int i = sw + it * kStrWaves;
+                wt[it] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(tail_address(i, i < n_items)));
+            }
+        }
+
+        // ---- whole panels: lane = row, a group is two 1 KiB loads; the wavefront takes groups sw, sw + 8, ...
+        if constexpr (MG > 0) {
+            const int gpw = (ng + kStrWaves - 1) / kStrWaves;   // groups per wavefront and panel
+            for (int pl = 0; pl < a.main_panels; ++pl) {
+                const int panel = pl * G + s_wg;
+                const int wsel = (panel >= a.ws.first[1]) + (panel >= a.ws.first[2]);
+                const int wpanel = panel - (wsel == 0 ? 0 : wsel == 1 ? a.ws.first[1] : a.ws.first[2]);
+                const uint8_t *codes = wsel == 0 ? a.ws.codes[0] : wsel == 1 ? a.ws.codes[1] : a.ws.codes[2];
+                const uint8_t *kmul = wsel == 0 ? a.ws.kmul[0] : wsel == 1 ? a.ws.kmul[1] : a.ws.kmul[2];
+                const int32_t fl = wsel == 0 ? f0 : wsel == 1 ? f1 : f2;
+                const uint8_t *pbase = codes + (size_t) wpanel * ng * 2048 + lane * 16;
+                int tot = 0;
+                for (int gi0 = 0; gi0 < gpw; gi0 += MG) {
+                    v4u w[MG][2];
+#pragma unroll
+                    for (int j = 0; j < MG; ++j) {
+                        int g = sw + (gi0 + j) * kStrWaves;
+                        if (g >= ng) g = 0;   // past the end: the first group again, contributes nothing
+                        w[j][0] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(pbase + (size_t) g * 2048));
+                        w[j][1] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(pbase + (size_t) g * 2048 + 1024));
+                    }
+                    if (!waited) {
+                        RQ_STAMP(2);
+                        wait_count(s_cnt, codes_ready);   // row in LDS, Sylvester passes, Paley, ranges, codes
+                        waited = true;
+                        RQ_STAMP(3);
+                    }
+#pragma unroll
+                    for (int j = 0; j < MG; ++j) {
+                        const int gq = sw + (gi0 + j) * kStrWaves;
+                        const bool on = gq < ng;
+                        const int g = on ? gq : 0;
+                        const uint4 a0 = *reinterpret_cast<const uint4 *>(s_act + g * 8);       // same address in every lane
+                        const uint4 a1 = *reinterpret_cast<const uint4 *>(s_act + g * 8 + 4);
+                        const int mzv = s_mz[g];
+                        int acc = 0, cs = 0;
+                        acc = dot8(w[j][0].x, a0.x, acc);
+                        acc = dot8(w[j][0].y, a0.y, acc);
+                        acc = dot8(w[j][0].z, a0.z, acc);
+                        acc = dot8(w[j][0].w, a0.w, acc);
+                        acc = dot8(w[j][1].x, a1.x, acc);
+                        acc = dot8(w[j][1].y, a1.y, acc);
+                        acc = dot8(w[j][1].z, a1.z, acc);
+                        acc = dot8(w[j][1].w, a1.w, acc);
+                        cs = dot8(w[j][0].x, 0x11111111u, cs);
+                        cs = dot8(w[j][0].y, 0x11111111u, cs);
+                        cs = dot8(w[j][0].z, 0x11111111u, cs);
+                        cs = dot8(w[j][0].w, 0x11111111u, cs);
+                        cs = dot8(w[j][1].x, 0x11111111u, cs);
+                        cs = dot8(w[j][1].y, 0x11111111u, cs);
+                        cs = dot8(w[j][1].z, 0x11111111u, cs);
+                        cs = dot8(w[j][1].w, 0x11111111u, cs);
+                        // |acc|, |cs * (8 - z)| <= 4096 and m <= 255: 24-bit multiplies are exact
+                        const int part = acc + __mul24((int) (int8_t) ((mzv >> 8) & 0xFF), cs);
+                        int term = __mul24(on ? (mzv & 0xFF) : 0, part);
+                        if (fl & 1) term *= (int) kmul[((size_t) wpanel * ng + g) * kPanelRows + lane];
+                        tot += term >> kTermShift;
+                    }
+                }
+                atomicAdd(&red[pl * kPanelRows + lane], tot);
+            }
+        }
+
+        // ---- remainder: lane = (row of the octet, half of the group, group of the item)
+        if constexpr (MT > 0) {
+            for (int i0 = 0; i0 < n_items || !waited; i0 += MT * kStrWaves) {
+                if (i0 > 0) {
+#pragma unroll
+                    for (int it = 0; it < MT; ++it) {
+                        const int i = i0 + sw + it * kStrWaves;
+                        wt[it] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(tail_address(i, i < n_items)));
+                    }
+                }
+                if (!waited) {
+                    RQ_STAMP(2);
+                    wait_count(s_cnt, codes_ready);
+                    waited = true;
+                    RQ_STAMP(3);
+                }
+#pragma unroll
+                for (int it = 0; it < MT; ++it) {
+                    const int iq = i0 + sw + it * kStrWaves;
+                    const bool on = iq < n_items;
+                    const int i = on ? iq : 0;
+                    const int ol = (int) (((uint32_t) i * (uint32_t) a.inv_nblk) >> 22);
+                    const int bb = i - ol * nblk;
+                    const int g = 4 * bb + g4;
+                    const uint4 av = *reinterpret_cast<const uint4 *>(s_act + g * 8 + 4 * h);
+                    const int mzv = s_mz[g];
+                    int acc = 0, cs = 0;
+                    acc = dot8(wt[it].x, av.x, acc);
+                    acc = dot8(wt[it].y, av.y, acc);
+                    acc = dot8(wt[it].z, av.z, acc);
+                    acc = dot8(wt[it].w, av.w, acc);
+                    cs = dot8(wt[it].x, 0x11111111u, cs);
+                    cs = dot8(wt[it].y, 0x11111111u, cs);
+                    cs = dot8(wt[it].z, 0x11111111u, cs);
+                    cs = dot8(wt[it].w, 0x11111111u, cs);
+                    int part = acc + __mul24((int) (int8_t) ((mzv >> 8) & 0xFF), cs);
+                    // the other half of the group sits eight lanes away in the same row of 16 lanes
+                    part += __builtin_amdgcn_update_dpp(0, part, 0x128 /* row_ror:8 */, 0xF, 0xF, false);
+                    int term = __mul24(mzv & 0xFF, part);
+                    if (anyk) {
+                        // weight multipliers (a format variant): fetched here, behind the stream
+                        const int o = oct0 + ol;
+                        const int panel = o >> 3;
+                        const int wsel = (panel >= a.ws.first[1]) + (panel >= a.ws.first[2]);
+                        const int32_t fl = wsel == 0 ? f0 : wsel == 1 ? f1 : f2;
+                        if (fl & 1) {
+                            const int wpanel = panel - (wsel == 0 ? 0 : wsel == 1 ? a.ws.first[1] : a.ws.first[2]);
+                            const uint8_t *kmul = wsel == 0 ? a.ws.kmul[0] : wsel == 1 ? a.ws.kmul[1] : a.ws.kmul[2];
+                            term *= (int) kmul[((size_t) wpanel * ng + g) * kPanelRows + (o & 7) * 8 + r8];
+                        }
+                    }
+                    term >>= kTermShift;
+                    // rows of a shared octet that belong to the neighbour land in cells that nobody writes out; items
+                    // past the end go to the spare cell
+                    if (h == 0) atomicAdd(&red[on ? main_cells + ol * 8 + r8 : kDecodeCells], term);
+                }
+            }
+        }
+        RQ_STAMP(4);
+        lds_barrier();   // all terms are in the cells
+        RQ_STAMP(5);
+    } else {
+        // =========================================================== the activation side (512 threads)
+        const int rt = tid;
+        int sync_target = 0;
+        // the row, 16 consecutive floats per thread and unit; all loads go out before the first barrier
+        constexpr int kUnits = 2;   // K <= 16384
+        float4 qv[kUnits][4];
+#pragma unroll
+        for (int ub = 0; ub < kUnits; ++ub) {
+            const int u = rt + ub * kRotThreads;
+            if (u < (K >> 4)) {
+                const float4 *src = reinterpret_cast<const float4 *>(a.x + 16 * u);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) qv[ub][j] = src[j];
+            }
+        }
+        // The stream starts only when the row has ARRIVED: requests queued behind the weight stream are served
+        // after it (a row requested just before the stream took 5 us instead of 1.5).
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        RQ_STAMP(1);
+#pragma unroll
+        for (int ub = 0; ub < kUnits; ++ub) {
+            const int u = rt + ub * kRotThreads;
+            if (u < (K >> 4)) {
+                float v[16] = { qv[ub][0].x, qv[ub][0].y, qv[ub][0].z, qv[ub][0].w, qv[ub][1].x, qv[ub][1].y,
+                                qv[ub][1].z, qv[ub][1].w, qv[ub][2].x, qv[ub][2].y, qv[ub][2].z, qv[ub][2].w,
+                                qv[ub][3].x, qv[ub][3].y, qv[ub][3].z, qv[ub][3].w };
+                if (a.rotate) {
+                    // Sylvester stages with strides 1, 2, 4, 8 in registers (chunks are multiples of 16 floats)
+#pragma unroll
+                    for (int hh = 1; hh < 16; hh <<= 1) {
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) {
+                            if ((j & hh) == 0) {
+                                const float lo = v[j], up = v[j + hh];
+                                v[j] = lo + up;
+                                v[j + hh] = lo - up;
+                            }
+                        }
+                    }
+                }
+                float *d = buf + padi(16 * u);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) d[j] = v[j];
+            }
+        }
+        rot_sync(s_cnt, sync_target, lane);
+        RQ_STAMP(2);
+
+        if (a.rotate) {
+            const int m = a.m;
+            const int lm = __ffs(m) - 1;
+            for (int ls = 4; ls < lm;) {
+                const int lr = lm - ls < 4 ? lm - ls : 4;
+                if (lr == 4) fwht_pass<4>(buf, K, lm, ls, rt, kRotThreads);
+                else if (lr == 3) fwht_pass<3>(buf, K, lm, ls, rt, kRotThreads);
+                else if (lr == 2) fwht_pass<2>(buf, K, lm, ls, rt, kRotThreads);
+                else fwht_pass<1>(buf, K, lm, ls, rt, kRotThreads);
+                ls += lr;
+                rot_sync(s_cnt, sync_target, lane);
+            }
+            RQ_STAMP(3);
+            if constexpr (P > 1) {
+                // Paley across the P chunks of every rotation block, into the second row buffer. A wave-item is
+                // (slice of kOut outputs, run of 64 columns); the slice's sign pattern is straight-line code.
+                constexpr int kOut = P / 4;
+                const int ncols = K / P;
+                const int pm = m + (m >> 4);
+                const int col_runs = (ncols + 63) >> 6;
+                const int n_it = 4 * col_runs;
+                const int per_wave = (n_it + kRotWaves - 1) / kRotWaves;
+                for (int it = 0; it < per_wave; ++it) {
+                    const int wi = wave * per_wave + it;
+                    if (wi >= n_it) break;
+                    const int s = wi / col_runs, cidx = (wi - s * col_runs) * 64 + lane;
+                    if (cidx >= ncols) continue;
+                    const int rb = cidx / m, j = cidx - rb * m;
+                    const int b0 = rb * a.n_rot + j;
+                    float col[P];
+                    const float *src = buf + padi(b0);
+#pragma unroll
+                    for (int i = 0; i < P; ++i) col[i] = src[i * pm];
+                    float out[kOut];
+                    paley_pick<P, kOut>(s, col, out);
+#pragma unroll
+                    for (int o = 0; o < kOut; ++o) alt[padi(b0 + (kOut * s + o) * m)] = out[o] * a.scale;
+                }
+                rot_sync(s_cnt, sync_target, lane);
+                buf = alt;
+            } else {
+                for (int i = rt; i < K; i += kRotThreads) buf[padi(i)] = buf[padi(i)] * a.scale;
+                rot_sync(s_cnt, sync_target, lane);
+            }
+        }
+
+        RQ_STAMP(4);
+        // ---- group ranges [min(x, 0), max(x, 0)] * clip and the token's widest range (reference lines 2646-2654):
+        // a thread per code word, eight lanes per group of 64
+        const int nw = K >> 3;
+        float rmax = 0.0f;
+        for (int w0 = 0; w0 < nw; w0 += kRotThreads) {
+            const int w = w0 + rt;
+            const bool on = w < nw;
+            float mn = 0.0f, mx = 0.0f;
+            if (on) {
+                const float *sp = buf + padi(8 * w);
+                const float4 v0 = make_float4(sp[0], sp[1], sp[2], sp[3]);
+                const float4 v1 = make_float4(sp[4], sp[5], sp[6], sp[7]);
+                mn = fminf(fminf(fminf(fminf(mn, v0.x), fminf(v0.y, v0.z)), fminf(fminf(v0.w, v1.x), fminf(v1.y, v1.z))), v1.w);
+                mx = fmaxf(fmaxf(fmaxf(fmaxf(mx, v0.x), fmaxf(v0.y, v0.z)), fmaxf(fmaxf(v0.w, v1.x), fmaxf(v1.y, v1.z))), v1.w);
+            }
+            mn = group8_reduce<false>(mn);
+            mx = group8_reduce<true>(mx);
+            const float lo = mn * a.clip, hi = mx * a.clip;
+            if (on) {
+                if ((rt & 7) == 0) {
+                    g_lo[w >> 3] = lo;
+                    g_hi[w >> 3] = hi;
+                }
+                rmax = fmaxf(rmax, hi - lo);
+            }
+        }
+        rmax = wave_max(rmax);
+        if (lane == 0) s_part[wave] = rmax;
+        rot_sync(s_cnt, sync_target, lane);
+        RQ_STAMP(5);
+
+        float R = s_part[0];
+#pragma unroll
+        for (int i = 1; i < kRotWaves; ++i) R = fmaxf(R, s_part[i]);
+        if (R == 0.0f) R = 2.0f;
+        const float u = R / 3825.0f;  // 15 * 255
+        if (rt == 0) s_unit[0] = u;
+
+        // ---- per group multiplier and zero point, per value code (reference lines 2662-2677)
+        for (int w0 = 0; w0 < nw; w0 += kRotThreads) {
+            const int w = w0 + rt;
+            if (w < nw) {
+                const int g = w >> 3;
+                const float lo = g_lo[g], hi = g_hi[g];
+                const int mg = (int) fminf(fmaxf(ceilf(((hi - lo) * 255.0f) / R), 1.0f), 255.0f);
+                const float inv = 1.0f / ((float) mg * u);
+                const float zf = fminf(fmaxf(rintf(-lo * inv), 0.0f), 15.0f);
+                const float *sp = buf + padi(8 * w);
+                const float f[8] = { sp[0], sp[1], sp[2], sp[3], sp[4], sp[5], sp[6], sp[7] };
+                uint32_t word = 0;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int q = (int) fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
+                    word |= (uint32_t) ((q - 8) & 0xF) << (4 * j);
+                }
+                s_act[w] = word;
+                if ((w & 7) == 0) s_mz[g] = mg | ((8 - (int) zf) & 0xFF) << 8;
+            }
+        }
+        rot_sync(s_cnt, sync_target, lane);   // codes, multipliers and unit are in LDS: the stream folds
+        RQ_STAMP(6);
+        lds_barrier();   // ... and has finished
+        RQ_STAMP(7);
+    }
+
+    // ---- epilogue (reference line 176): three fp32 multiplies in the reference's order
+    if (y_row != nullptr) *y_row = (((float) red[tid] * 16.0f) * s_unit[0]) * pre_sw;
+}
+
+template <int P, int MG, int MT>
+hipError_t launch_pmt(const DecodeKernelArgs &k, int grid, size_t lds, hipStream_t stream) {
+    static bool attr_set = false;   // (also done per device by init_decode_kernels)
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_decode_kernel<P, MG, MT>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((rq_decode_kernel<P, MG, MT>), dim3(grid), dim3(kDecThreads), lds, stream, k);
+    return hipGetLastError();
+}
+
+// whole panels: 10 groups per wavefront and round cover K = 5120 in one round (12: K = 6144); the remainder gets 4
+// items per wavefront and round beside whole panels, 12 when the launch is remainder only
+template <int P>
+hipError_t launch_p(const DecodeKernelArgs &k, int grid, size_t lds, hipStream_t stream) {
+    if (k.main_panels == 0) return launch_pmt<P, 0, 12>(k, grid, lds, stream);
+    const int gpw = (k.K / kGroup + kStrWaves - 1) / kStrWaves;
+    const bool tail = k.q_base > 0 || k.q_extra > 0;
+    if (gpw % 12 == 0 || (gpw % 10 != 0 && gpw > 10)) {
+        return tail ? launch_pmt<P, 12, 2>(k, grid, lds, stream) : launch_pmt<P, 12, 0>(k, grid, lds, stream);
+    }
+    return tail ? launch_pmt<P, 10, 4>(k, grid, lds, stream) : launch_pmt<P, 10, 0>(k, grid, lds, stream);
+}
+
+template <int P, int MG, int MT>
+hipError_t allow_lds() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_decode_kernel<P, MG, MT>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
+}
+
+template <int P>
+hipError_t allow_lds_p() {
+    hipError_t e = allow_lds<P, 0, 12>();
+    if (e == hipSuccess) e = allow_lds<P, 10, 4>();
+    if (e == hipSuccess) e = allow_lds<P, 10, 0>();
+    if (e == hipSuccess) e = allow_lds<P, 12, 2>();
+    if (e == hipSuccess) e = allow_lds<P, 12, 0>();
+    return e;
+}
+
+}  // namespace
+
+hipError_t init_decode_kernels() {
+    hipError_t e = allow_lds_p<1>();
+    if (e == hipSuccess) e = allow_lds_p<12>();
+    if (e == hipSuccess) e = allow_lds_p<20>();
+    return e;
+}
+
+// Which one-token problems the single-launch kernel takes: activation groups of 64, a rotation with a short Paley
+// stage whose chunks are multiples of 16 floats (or no rotation), and a row that fits LDS twice.
+bool decode_takes(int K, int rotate, int p, int m, int act_group) {
+    if (act_group != kGroup) return false;
+    if (K > 16384) return false;
+    if (rotate) {
+        if (p != 1 && p != 12 && p != 20) return false;
+        if ((m & 15) != 0) return false;
+    }
+    return decode_lds_bytes(K, rotate && p > 1) <= 160 * 1024 - 64;
+}
+
+hipError_t launch_decode(const DecodeArgs &d, hipStream_t stream) {
+    DecodeKernelArgs k;
+    k.ws = make_weight_set(d.w);
+    k.x = d.x;
+    k.K = d.K;
+    k.rotate = d.rotate;
+    k.n_rot = d.n_rot;
+    k.m = d.m;
+    k.scale = d.scale;
+    k.clip = d.clip;
+    k.inv_nblk = (1 << 22) / (d.K / 256) + 1;
+    const int lm = d.rotate ? __builtin_ctz((unsigned) d.m) : 0;
+    k.n_pass = d.rotate && lm > 4 ? (lm - 4 + 3) / 4 : 0;
+    const int n_panels = k.ws.first[kMaxFused];
+    // one workgroup per compute unit: whole panels as far as they go round, the remainder in quads of rows. More
+    // workgroups (a multiple of the compute units) only when the rows of one would not fit its LDS cells.
+    const int cus = d.compute_units > 0 ? d.compute_units : 256;
+    int grid = cus;
+    for (;;) {
+        const int mp = n_panels / grid;
+        const int tail_quads = (n_panels - mp * grid) * 16;
+        const int octets = tail_quads ? (tail_quads + grid - 1) / grid / 2 + 2 : 0;
+        if (mp * kPanelRows + octets * 8 <= kDecodeCells) break;
+        grid += cus;
+    }
+    if (grid > n_panels * 16) grid = n_panels * 16;
+    k.main_panels = n_panels / grid;
+    k.tail_panel0 = k.main_panels * grid;
+    const int tail_quads = (n_panels - k.tail_panel0) * 16;
+    k.q_base = tail_quads / grid;
+    k.q_extra = tail_quads % grid;
+    const size_t lds = decode_lds_bytes(d.K, d.rotate && d.p > 1);
+    switch (d.rotate ? d.p : 1) {
+        case 1:  return launch_p<1>(k, grid, lds, stream);
+        case 12: return launch_p<12>(k, grid, lds, stream);
+        case 20: return launch_p<20>(k, grid, lds, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace rq
