@@ -26,13 +26,20 @@
 #pragma clang fp contract(off)
 
 #ifdef RQ_DECODE_TIMING
+// Phase timestamps of workgroup 0 (wavefronts 0 and 8), kept in registers and written out at the very end: a store in
+// the middle of the kernel would queue behind the weight stream and distort what it measures.
 __device__ unsigned long long rq_decode_stamps[64];
-#define RQ_STAMP(i) do { if (blockIdx.x == 0 && (threadIdx.x == 0 || threadIdx.x == 512)) rq_decode_stamps[(i) + (threadIdx.x ? 32 : 0)] = __builtin_readcyclecounter(); } while (0)
+#define RQ_STAMP_DECL unsigned long long rq_st[8] = {}
+#define RQ_STAMP(i) do { rq_st[(i)] = __builtin_readcyclecounter(); } while (0)
+#define RQ_STAMP_FLUSH do { if (blockIdx.x == 0 && (threadIdx.x == 0 || threadIdx.x == 512)) { \
+        for (int i_ = 0; i_ < 8; ++i_) rq_decode_stamps[i_ + (threadIdx.x ? 32 : 0)] = rq_st[i_]; } } while (0)
 extern "C" int rq_w4a4_decode_stamps(unsigned long long *out) {
     return (int) hipMemcpyFromSymbol(out, HIP_SYMBOL(rq_decode_stamps), sizeof(rq_decode_stamps));
 }
 #else
+#define RQ_STAMP_DECL do { } while (0)
 #define RQ_STAMP(i) do { } while (0)
+#define RQ_STAMP_FLUSH do { } while (0)
 #endif
 
 namespace rq {
@@ -71,16 +78,33 @@ __device__ __forceinline__ int align4(int v) { return (v + 3) & ~3; }
 // (The counter is read through an LDS-typed pointer: a generic one makes the poll a FLAT load, which queues behind
 // the weight stream.)
 typedef __attribute__((address_space(3))) int lds_int;
+// One Sylvester stage between lanes: `ctrl` swaps every lane with its partner (the lane whose unit differs in the
+// stage's index bit); the lane of the lower unit gets a + b, the upper one a - b with a the lower unit's value
+// (reference lines 2454-2464). t - v is formed as t + (-v): the same IEEE operation.
+template <int CTRL>
+__device__ __forceinline__ void dpp_stage(float (&v)[16], uint32_t upper_sign) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const float t = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v[j]), CTRL,
+                                                                              0xF, 0xF, false));
+        const float sv = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v[j]) ^ upper_sign);
+        v[j] = t + sv;
+    }
+}
+
+template <bool SLEEP>
 __device__ __forceinline__ void wait_count(const int *cnt, int target) {
     const volatile lds_int *c = (const volatile lds_int *) cnt;
-    while (__builtin_amdgcn_readfirstlane(*c) < target) __builtin_amdgcn_s_sleep(1);
+    while (__builtin_amdgcn_readfirstlane(*c) < target) {
+        if (SLEEP) __builtin_amdgcn_s_sleep(2);   // the stream waits for microseconds; the rotation for a straggler
+    }
     asm volatile("" ::: "memory");
 }
 __device__ __forceinline__ void rot_sync(int *cnt, int &target, int lane) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     if (lane == 0) atomicAdd(cnt, 1);
     target += kRotWaves;
-    wait_count(cnt, target);
+    wait_count<false>(cnt, target);
 }
 
 // LDS: [row][row (Paley output)][g_lo][g_hi][codes][mz][cells][wave maxima, unit]
@@ -97,6 +121,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
     extern __shared__ __align__(16) float smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    RQ_STAMP_DECL;
     RQ_STAMP(0);
     const int K = a.K, ng = K / kGroup;
     const int Kp = align4(padi(K) + 1);
@@ -165,7 +190,13 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         const int32_t f1 = __builtin_nontemporal_load(a.ws.flags[1]);
         const int32_t f2 = __builtin_nontemporal_load(a.ws.flags[2]);
 
-        __builtin_amdgcn_s_barrier();   // the rotate wavefronts have the row
+        // Behind this barrier the rotate wavefronts have the row. Not one weight is requested before: with 2 (4) of a
+        // wavefront's 22 loads ahead of the barrier the row arrived later and the whole call took 12.0 (12.5) us
+        // instead of 11.2.
+        // Behind this barrier the rotate wavefronts have the row. Not one weight is requested before: with 1, 2, 4
+        // or 9 of a wavefront's 10 groups ahead of the barrier the row arrives later and the whole call takes 11.9,
+        // 11.7, 12.5 and 15.3 us instead of 11.0.
+        __builtin_amdgcn_s_barrier();
         RQ_STAMP(1);
 
         const bool anyk = ((f0 | f1 | f2) & 1) != 0;
@@ -219,27 +250,42 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                     }
                     if (!waited) {
                         RQ_STAMP(2);
-                        wait_count(s_cnt, codes_ready);   // row in LDS, Sylvester passes, Paley, ranges, codes
+                        wait_count<true>(s_cnt, codes_ready);   // row in LDS, Sylvester passes, Paley, ranges, codes
                         waited = true;
                         RQ_STAMP(3);
+                    }
+                    // The activation words of a group are the same for all 64 rows. The wavefront's MG groups are
+                    // MG x 8 code words and MG (m, z) words: fetched from LDS once, one word per lane, and handed to
+                    // the dot products as scalars (v_readlane), so the fold of a group waits for no LDS round trip.
+                    uint32_t aw[2];
+                    int mzw;
+                    {
+                        const int gl = sw + (gi0 + (lane >> 3)) * kStrWaves, gh = sw + (gi0 + 8 + (lane >> 3)) * kStrWaves;
+                        aw[0] = s_act[(gl < ng ? gl : 0) * 8 + (lane & 7)];
+                        aw[1] = MG > 8 ? s_act[(gh < ng && lane < (MG - 8) * 8 ? gh : 0) * 8 + (lane & 7)] : 0u;
+                        const int gm = sw + (gi0 + lane) * kStrWaves;
+                        mzw = s_mz[gm < ng && lane < MG ? gm : 0];
                     }
 #pragma unroll
                     for (int j = 0; j < MG; ++j) {
                         const int gq = sw + (gi0 + j) * kStrWaves;
                         const bool on = gq < ng;
                         const int g = on ? gq : 0;
-                        const uint4 a0 = *reinterpret_cast<const uint4 *>(s_act + g * 8);       // same address in every lane
-                        const uint4 a1 = *reinterpret_cast<const uint4 *>(s_act + g * 8 + 4);
-                        const int mzv = s_mz[g];
+                        uint32_t av[8];
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) {
+                            av[i] = (uint32_t) __builtin_amdgcn_readlane((int) aw[(j * 8 + i) >> 6], (j * 8 + i) & 63);
+                        }
+                        const int mzv = __builtin_amdgcn_readlane(mzw, j);
                         int acc = 0, cs = 0;
-                        acc = dot8(w[j][0].x, a0.x, acc);
-                        acc = dot8(w[j][0].y, a0.y, acc);
-                        acc = dot8(w[j][0].z, a0.z, acc);
-                        acc = dot8(w[j][0].w, a0.w, acc);
-                        acc = dot8(w[j][1].x, a1.x, acc);
-                        acc = dot8(w[j][1].y, a1.y, acc);
-                        acc = dot8(w[j][1].z, a1.z, acc);
-                        acc = dot8(w[j][1].w, a1.w, acc);
+                        acc = dot8(w[j][0].x, av[0], acc);
+                        acc = dot8(w[j][0].y, av[1], acc);
+                        acc = dot8(w[j][0].z, av[2], acc);
+                        acc = dot8(w[j][0].w, av[3], acc);
+                        acc = dot8(w[j][1].x, av[4], acc);
+                        acc = dot8(w[j][1].y, av[5], acc);
+                        acc = dot8(w[j][1].z, av[6], acc);
+                        acc = dot8(w[j][1].w, av[7], acc);
                         cs = dot8(w[j][0].x, 0x11111111u, cs);
                         cs = dot8(w[j][0].y, 0x11111111u, cs);
                         cs = dot8(w[j][0].z, 0x11111111u, cs);
@@ -271,7 +317,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                 }
                 if (!waited) {
                     RQ_STAMP(2);
-                    wait_count(s_cnt, codes_ready);
+                    wait_count<true>(s_cnt, codes_ready);
                     waited = true;
                     RQ_STAMP(3);
                 }
@@ -324,12 +370,21 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         // =========================================================== the activation side (512 threads)
         const int rt = tid;
         int sync_target = 0;
-        // the row, 16 consecutive floats per thread and unit; all loads go out before the first barrier
+        // the row, 16 consecutive floats per thread and unit; all loads go out before the first barrier.
+        // Chunks of 256 floats (16 units): the 16 lanes of a DPP row hold one chunk, so the Sylvester stages with
+        // strides 16 .. 128 run between lanes and the row makes no trip through LDS between its stages. Lane l of a row
+        // holds the unit whose index bits (b0, b1, b2, b3) give l = b0 ^ 2 b1 ^ 7 b2 ^ 8 b3: the partners of the four
+        // stages are then l ^ 1, l ^ 2, l ^ 7, l ^ 8, which are single DPP controls.
+        const bool dpp256 = a.rotate && a.m == 256;
+        const int lr = lane & 15;
+        const int hb3 = lr >> 3, hr = lr & 7, hb2 = hr >> 2, hr2 = hr ^ (hb2 ? 7 : 0);
+        const int unit_of_lane = (hr2 & 1) | (hr2 & 2) | hb2 << 2 | hb3 << 3;
         constexpr int kUnits = 2;   // K <= 16384
         float4 qv[kUnits][4];
 #pragma unroll
         for (int ub = 0; ub < kUnits; ++ub) {
-            const int u = rt + ub * kRotThreads;
+            int u = rt + ub * kRotThreads;
+            if (dpp256) u = (u & ~15) | unit_of_lane;
             if (u < (K >> 4)) {
                 const float4 *src = reinterpret_cast<const float4 *>(a.x + 16 * u);
 #pragma unroll
@@ -343,8 +398,9 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         RQ_STAMP(1);
 #pragma unroll
         for (int ub = 0; ub < kUnits; ++ub) {
-            const int u = rt + ub * kRotThreads;
-            if (u < (K >> 4)) {
+            int u = rt + ub * kRotThreads;
+            if (dpp256) u = (u & ~15) | unit_of_lane;
+            if (u < (K >> 4)) {   // (whole DPP rows: K / 16 is a multiple of 16 when the chunks are 256 long)
                 float v[16] = { qv[ub][0].x, qv[ub][0].y, qv[ub][0].z, qv[ub][0].w, qv[ub][1].x, qv[ub][1].y,
                                 qv[ub][1].z, qv[ub][1].w, qv[ub][2].x, qv[ub][2].y, qv[ub][2].z, qv[ub][2].w,
                                 qv[ub][3].x, qv[ub][3].y, qv[ub][3].z, qv[ub][3].w };
@@ -362,6 +418,12 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                         }
                     }
                 }
+                if (dpp256) {
+                    dpp_stage<0xB1>(v, (uint32_t) (hr2 & 1) << 31);          // stride 16: quad_perm [1, 0, 3, 2]
+                    dpp_stage<0x4E>(v, (uint32_t) ((hr2 >> 1) & 1) << 31);   // stride 32: quad_perm [2, 3, 0, 1]
+                    dpp_stage<0x141>(v, (uint32_t) hb2 << 31);               // stride 64: row_half_mirror
+                    dpp_stage<0x128>(v, (uint32_t) hb3 << 31);               // stride 128: row_ror:8
+                }
                 float *d = buf + padi(16 * u);
 #pragma unroll
                 for (int j = 0; j < 16; ++j) d[j] = v[j];
@@ -373,14 +435,16 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         if (a.rotate) {
             const int m = a.m;
             const int lm = __ffs(m) - 1;
-            for (int ls = 4; ls < lm;) {
-                const int lr = lm - ls < 4 ? lm - ls : 4;
-                if (lr == 4) fwht_pass<4>(buf, K, lm, ls, rt, kRotThreads);
-                else if (lr == 3) fwht_pass<3>(buf, K, lm, ls, rt, kRotThreads);
-                else if (lr == 2) fwht_pass<2>(buf, K, lm, ls, rt, kRotThreads);
-                else fwht_pass<1>(buf, K, lm, ls, rt, kRotThreads);
-                ls += lr;
-                rot_sync(s_cnt, sync_target, lane);
+            if (!dpp256) {
+                for (int ls = 4; ls < lm;) {
+                    const int lr2 = lm - ls < 4 ? lm - ls : 4;
+                    if (lr2 == 4) fwht_pass<4>(buf, K, lm, ls, rt, kRotThreads);
+                    else if (lr2 == 3) fwht_pass<3>(buf, K, lm, ls, rt, kRotThreads);
+                    else if (lr2 == 2) fwht_pass<2>(buf, K, lm, ls, rt, kRotThreads);
+                    else fwht_pass<1>(buf, K, lm, ls, rt, kRotThreads);
+                    ls += lr2;
+                    rot_sync(s_cnt, sync_target, lane);
+                }
             }
             RQ_STAMP(3);
             if constexpr (P > 1) {
@@ -395,18 +459,30 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                 for (int it = 0; it < per_wave; ++it) {
                     const int wi = wave * per_wave + it;
                     if (wi >= n_it) break;
-                    const int s = wi / col_runs, cidx = (wi - s * col_runs) * 64 + lane;
+                    const int s = (wi >= col_runs) + (wi >= 2 * col_runs) + (wi >= 3 * col_runs);   // wi / col_runs
+                    const int cidx = (wi - s * col_runs) * 64 + lane;
                     if (cidx >= ncols) continue;
-                    const int rb = cidx / m, j = cidx - rb * m;
+                    const int rb = cidx >> lm, j = cidx & (m - 1);   // chunk lengths are powers of two
                     const int b0 = rb * a.n_rot + j;
                     float col[P];
                     const float *src = buf + padi(b0);
-#pragma unroll
-                    for (int i = 0; i < P; ++i) col[i] = src[i * pm];
                     float out[kOut];
-                    paley_pick<P, kOut>(s, col, out);
+                    if (m == 256) {
+                        // chunks of 256: the chunk stride in the padded row is the constant 272, so the P loads and the
+                        // kOut stores are immediate offsets from one address
 #pragma unroll
-                    for (int o = 0; o < kOut; ++o) alt[padi(b0 + (kOut * s + o) * m)] = out[o] * a.scale;
+                        for (int i = 0; i < P; ++i) col[i] = src[i * 272];
+                        paley_pick<P, kOut>(s, col, out);
+                        float *dst = alt + padi(b0) + kOut * s * 272;
+#pragma unroll
+                        for (int o = 0; o < kOut; ++o) dst[o * 272] = out[o] * a.scale;
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < P; ++i) col[i] = src[i * pm];
+                        paley_pick<P, kOut>(s, col, out);
+#pragma unroll
+                        for (int o = 0; o < kOut; ++o) alt[padi(b0 + (kOut * s + o) * m)] = out[o] * a.scale;
+                    }
                 }
                 rot_sync(s_cnt, sync_target, lane);
                 buf = alt;
@@ -418,29 +494,29 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
 
         RQ_STAMP(4);
         // ---- group ranges [min(x, 0), max(x, 0)] * clip and the token's widest range (reference lines 2646-2654):
-        // a thread per code word, eight lanes per group of 64
+        // a thread per code word, eight lanes per group of 64; the word's eight values stay in registers for the codes
         const int nw = K >> 3;
+        constexpr int kWordRounds = 4;   // K <= 16384
+        float f[kWordRounds][8];
+        float g_lo_r[kWordRounds], g_hi_r[kWordRounds];
         float rmax = 0.0f;
-        for (int w0 = 0; w0 < nw; w0 += kRotThreads) {
-            const int w = w0 + rt;
-            const bool on = w < nw;
-            float mn = 0.0f, mx = 0.0f;
-            if (on) {
-                const float *sp = buf + padi(8 * w);
-                const float4 v0 = make_float4(sp[0], sp[1], sp[2], sp[3]);
-                const float4 v1 = make_float4(sp[4], sp[5], sp[6], sp[7]);
-                mn = fminf(fminf(fminf(fminf(mn, v0.x), fminf(v0.y, v0.z)), fminf(fminf(v0.w, v1.x), fminf(v1.y, v1.z))), v1.w);
-                mx = fmaxf(fmaxf(fmaxf(fmaxf(mx, v0.x), fmaxf(v0.y, v0.z)), fmaxf(fmaxf(v0.w, v1.x), fmaxf(v1.y, v1.z))), v1.w);
-            }
-            mn = group8_reduce<false>(mn);
-            mx = group8_reduce<true>(mx);
-            const float lo = mn * a.clip, hi = mx * a.clip;
-            if (on) {
-                if ((rt & 7) == 0) {
-                    g_lo[w >> 3] = lo;
-                    g_hi[w >> 3] = hi;
-                }
-                rmax = fmaxf(rmax, hi - lo);
+#pragma unroll
+        for (int wr = 0; wr < kWordRounds; ++wr) {
+            const int w = wr * kRotThreads + rt;
+            if (wr * kRotThreads < nw) {   // uniform
+                const bool on = w < nw;
+                const float *sp = buf + padi(8 * (on ? w : 0));
+#pragma unroll
+                for (int j = 0; j < 8; ++j) f[wr][j] = on ? sp[j] : 0.0f;
+                float mn = fminf(fminf(fminf(fminf(0.0f, f[wr][0]), fminf(f[wr][1], f[wr][2])),
+                                       fminf(fminf(f[wr][3], f[wr][4]), fminf(f[wr][5], f[wr][6]))), f[wr][7]);
+                float mx = fmaxf(fmaxf(fmaxf(fmaxf(0.0f, f[wr][0]), fmaxf(f[wr][1], f[wr][2])),
+                                       fmaxf(fmaxf(f[wr][3], f[wr][4]), fmaxf(f[wr][5], f[wr][6]))), f[wr][7]);
+                mn = group8_reduce<false>(mn);
+                mx = group8_reduce<true>(mx);
+                g_lo_r[wr] = mn * a.clip;
+                g_hi_r[wr] = mx * a.clip;
+                if (on) rmax = fmaxf(rmax, g_hi_r[wr] - g_lo_r[wr]);
             }
         }
         rmax = wave_max(rmax);
@@ -456,24 +532,22 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         if (rt == 0) s_unit[0] = u;
 
         // ---- per group multiplier and zero point, per value code (reference lines 2662-2677)
-        for (int w0 = 0; w0 < nw; w0 += kRotThreads) {
-            const int w = w0 + rt;
-            if (w < nw) {
-                const int g = w >> 3;
-                const float lo = g_lo[g], hi = g_hi[g];
+#pragma unroll
+        for (int wr = 0; wr < kWordRounds; ++wr) {
+            const int w = wr * kRotThreads + rt;
+            if (wr * kRotThreads < nw && w < nw) {
+                const float lo = g_lo_r[wr], hi = g_hi_r[wr];
                 const int mg = (int) fminf(fmaxf(ceilf(((hi - lo) * 255.0f) / R), 1.0f), 255.0f);
                 const float inv = 1.0f / ((float) mg * u);
                 const float zf = fminf(fmaxf(rintf(-lo * inv), 0.0f), 15.0f);
-                const float *sp = buf + padi(8 * w);
-                const float f[8] = { sp[0], sp[1], sp[2], sp[3], sp[4], sp[5], sp[6], sp[7] };
                 uint32_t word = 0;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const int q = (int) fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f);
+                    const int q = (int) fminf(fmaxf(rintf(f[wr][j] * inv) + zf, 0.0f), 15.0f);
                     word |= (uint32_t) ((q - 8) & 0xF) << (4 * j);
                 }
                 s_act[w] = word;
-                if ((w & 7) == 0) s_mz[g] = mg | ((8 - (int) zf) & 0xFF) << 8;
+                if ((w & 7) == 0) s_mz[w >> 3] = mg | ((8 - (int) zf) & 0xFF) << 8;
             }
         }
         rot_sync(s_cnt, sync_target, lane);   // codes, multipliers and unit are in LDS: the stream folds
@@ -484,6 +558,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
 
     // ---- epilogue (reference line 176): three fp32 multiplies in the reference's order
     if (y_row != nullptr) *y_row = (((float) red[tid] * 16.0f) * s_unit[0]) * pre_sw;
+    RQ_STAMP_FLUSH;
 }
 
 template <int P, int MG, int MT>
@@ -561,7 +636,7 @@ hipError_t launch_decode(const DecodeArgs &d, hipStream_t stream) {
     k.clip = d.clip;
     k.inv_nblk = (1 << 22) / (d.K / 256) + 1;
     const int lm = d.rotate ? __builtin_ctz((unsigned) d.m) : 0;
-    k.n_pass = d.rotate && lm > 4 ? (lm - 4 + 3) / 4 : 0;
+    k.n_pass = d.rotate && lm > 4 && d.m != 256 ? (lm - 4 + 3) / 4 : 0;   // chunks of 256: the stages run between lanes
     const int n_panels = k.ws.first[kMaxFused];
     // one workgroup per compute unit: whole panels as far as they go round, the remainder in quads of rows. More
     // workgroups (a multiple of the compute units) only when the rows of one would not fit its LDS cells.
