@@ -46,10 +46,8 @@ namespace {
 struct Env {
     float clip[2];   // RQ_ACT_CLIP, RQ_ACT_CLIP_H (falls back to the former); -1 = unset
     int   act_group;
-    int   gemm_min;  // smallest token count that takes the tiled MFMA GEMM
-    int   gemv_max;  // largest token count that takes the GEMV; between the two: the skinny MFMA kernel
-    int   skinny_single;  // skinny path: single-plane activations (RQ_SKINNY_SINGLE=0 switches back to two digits)
-    int   decode_fused;   // one token: the single-launch kernel (RQ_DECODE_FUSED=0: rotation kernel + GEMV)
+    int   decode_fused;   // one token: the single-launch kernel. RQ_DECODE_FUSED=0 (the one debug switch of the
+                          // library) sends one token down the rotation kernel + GEMV that serves two and three
     Env() {
         const char *e = getenv("RQ_ACT_CLIP");
         const char *eh = getenv("RQ_ACT_CLIP_H");
@@ -58,16 +56,6 @@ struct Env {
         const char *g = getenv("RQ_ACT_GROUP");
         const int v = g ? atoi(g) : 64;
         act_group = v == 128 || v == 256 ? v : 64;
-        const char *gm = getenv("RQ_GEMM_MIN");
-        gemm_min = gm ? atoi(gm) : kSkinnyTokens + 1;
-        if (gemm_min < 1) gemm_min = 1;
-        if (gemm_min > kSkinnyTokens + 1) gemm_min = kSkinnyTokens + 1;
-        const char *gv = getenv("RQ_GEMV_MAX");
-        gemv_max = gv ? atoi(gv) : 3;   // measured: from four tokens on the skinny MFMA kernel is the faster op
-        if (gemv_max < 0) gemv_max = 0;
-        if (gemv_max > kGemvMaxTokens) gemv_max = kGemvMaxTokens;
-        const char *ss = getenv("RQ_SKINNY_SINGLE");
-        skinny_single = ss ? atoi(ss) != 0 : 1;
         const char *df = getenv("RQ_DECODE_FUSED");
         decode_fused = df ? atoi(df) != 0 : 1;
     }
@@ -105,21 +93,6 @@ void *static_scratch(hipError_t *err) {
     return ptr[dev];
 }
 
-// Compute units of the current device, read once per device (first use of a weight; a later call only looks it up).
-int device_compute_units() {
-    static std::mutex mu;
-    static int cus[kMaxDevices] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
-    std::lock_guard<std::mutex> lock(mu);
-    if (cus[dev] == 0) {
-        int v = 0;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) return 0;
-        cus[dev] = v;
-    }
-    return cus[dev];
-}
-
 bool is_w_type(int type) { return type == RQ_TYPE_W4A4 || type == RQ_TYPE_W4A4H; }
 
 bool shape_ok(int type, int64_t K, int64_t N, int64_t M) {
@@ -139,10 +112,13 @@ bool rotation_of(int type, int64_t K, int64_t n_rot, int &p, int &m) {
     return hadamard_factor(n_rot, p, m);
 }
 
+// Measured crossovers (K = 5120, N = 17408): up to three tokens the dot-product GEMV, from four the skinny MFMA
+// kernel, from 65 the tiled MFMA GEMM.
 enum Path { kPathGemv, kPathSkinny, kPathGemm };
+constexpr int kGemvMax = 3;
 Path path_of(int64_t M) {
-    if (M >= env().gemm_min) return kPathGemm;
-    return M <= env().gemv_max ? kPathGemv : kPathSkinny;
+    if (M > kSkinnyTokens) return kPathGemm;
+    return M <= kGemvMax ? kPathGemv : kPathSkinny;
 }
 
 int run_products(int type, int n, const void *const *prepared, int64_t K, const int64_t *N, const float *x,
@@ -237,7 +213,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     q.Mp = act_mp;
     // the skinny path: one plane of q - z and the multipliers beside it (half the activation bytes per group, which
     // count against the weight bytes a compute unit can have in flight)
-    const bool single = path == kPathSkinny && env().skinny_single;
+    const bool single = path == kPathSkinny;
     q.single = single;
     q.mvals = reinterpret_cast<uint8_t *>(wsb + W.off_i8) + (size_t) (K / kGroup) * act_mp * 64;
     const float *gemv_x = x;      // what the GEMV quantizes from: the rotated rows, or x itself for W4A4
@@ -333,6 +309,21 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
 }
 
 }  // namespace
+
+int device_compute_units() {
+    static std::mutex mu;
+    static int cus[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    std::lock_guard<std::mutex> lock(mu);
+    if (cus[dev] == 0) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+        cus[dev] = v;
+    }
+    return cus[dev];
+}
+
 }  // namespace rq
 
 using namespace rq;

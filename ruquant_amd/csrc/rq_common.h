@@ -259,6 +259,13 @@ hipError_t launch_decode(const DecodeArgs &a, hipStream_t stream);
 hipError_t init_decode_kernels();
 bool decode_takes(int K, int rotate, int p, int m, int act_group);
 
+// Compute units of the current device, read once per device (hipDeviceAttributeMultiprocessorCount); 256 when the
+// runtime will not say. The launch plans count rounds of the chip with it.
+int device_compute_units();
+// XCDs (accelerator dies, each with its own L2) that workgroups are dealt to round robin: 8 on MI355X. Used only to
+// place workgroups that share operands on one L2; a different count costs locality, never correctness.
+constexpr int kXcds = 8;
+
 hipError_t launch_prepare(const void *blocks, const PreparedLayout &L, uint8_t *prepared, hipStream_t stream);
 
 bool hadamard_factor(int64_t n, int &p, int &m);

@@ -142,7 +142,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
     const int G = gridDim.x;
     const int s_wg = blockIdx.x;
     int slot = s_wg;
-    if ((G & 7) == 0) slot = (int) (blockIdx.x & 7) * (G >> 3) + (int) (blockIdx.x >> 3);
+    if (G % kXcds == 0) slot = (int) (blockIdx.x % kXcds) * (G / kXcds) + (int) (blockIdx.x / kXcds);
     const int q0 = a.tail_panel0 * 16 + slot * a.q_base + (slot < a.q_extra ? slot : a.q_extra);
     const int q1 = q0 + a.q_base + (slot < a.q_extra ? 1 : 0);
     const int oct0 = q0 >> 1, n_oct = q1 > q0 ? ((q1 + 1) >> 1) - oct0 : 0;

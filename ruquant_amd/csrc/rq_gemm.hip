@@ -373,8 +373,8 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     int row_tile, t0;
     if (!NARROW) {
         int v = blockIdx.x;
-        const int per_xcd = n_tiles / 8;
-        if (v < per_xcd * 8) v = (v & 7) * per_xcd + (v >> 3);
+        const int per_xcd = n_tiles / kXcds;
+        if (v < per_xcd * kXcds) v = (v % kXcds) * per_xcd + v / kXcds;
         if (gs) {
             // (wide tiles only: gs carries the flag) super-tiles of 8 row tiles x 4 token tiles = the 32 workgroups an
             // XCD runs at a time: together they read 8 weight tiles and 4 activation tiles, the mix that puts the
@@ -393,8 +393,8 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
         // tokens are enumerated (an empty workgroup would still take a slot of the round-robin dispatch). Each XCD
         // gets a contiguous run, so the quarters of one row tile share its weights in one L2.
         int b = blockIdx.x;
-        const int per_xcd = n_tiles / 8;          // here: number of narrow workgroups
-        if (b < per_xcd * 8) b = (b & 7) * per_xcd + (b >> 3);
+        const int per_xcd = n_tiles / kXcds;          // here: number of narrow workgroups
+        if (b < per_xcd * kXcds) b = (b % kXcds) * per_xcd + b / kXcds;
         const int per_row = 4 * (n_tok_tiles - 1) + live_last;
         const int r = b / per_row, slot = b - r * per_row;
         row_tile = first_tile / n_tok_tiles + r;
@@ -520,11 +520,10 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     const int n_row_tiles = (a.L.n_panels + 3) / 4;
     const int n_tok_tiles = a.Mp / kBT;
     const int n_tiles = n_row_tiles * n_tok_tiles;
-    static const int force = getenv("RQ_GEMM_NARROW") ? atoi(getenv("RQ_GEMM_NARROW")) : -1;   // 0: never, 1: always
     // How many tiles run wide. A round of 256 wide tiles takes about 2.6 times a round of 256 narrow ones (a
     // quarter of the work each, at two thirds of the efficiency); rounds are whole. Candidates: all narrow, whole
     // wide rounds (in whole row tiles) with a narrow tail, all wide.
-    const int kCUs = 256;
+    const int kCUs = device_compute_units();
     const int live_last = ((a.M + kBTn - 1) / kBTn + 3) % 4 + 1;     // token quarters of the last tile that hold tokens
     const int per_row = 4 * (n_tok_tiles - 1) + live_last;           // narrow workgroups per row tile
     auto cost = [&](int nw) {                                        // nw: a multiple of n_tok_tiles (whole row tiles)
@@ -535,18 +534,16 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     const int whole = n_tiles / kCUs * kCUs / n_tok_tiles * n_tok_tiles;
     if (cost(whole) < cost(n_wide)) n_wide = whole;
     if (cost(n_tiles) < cost(n_wide)) n_wide = n_tiles;
-    if (force == 0) n_wide = n_tiles;
-    if (force == 1 || a.groups_per_fold > 1) n_wide = 0;   // wider activation groups: narrow tiles only
+    if (a.groups_per_fold > 1) n_wide = 0;   // wider activation groups: narrow tiles only
     // A third way to run the rows that the whole wide rounds leave over: the skinny kernel (rq_skinny.hip), a
     // workgroup per panel of 64 rows and block of 32 tokens, whole K, no LDS staging. A round of 256 of those takes
     // about 0.65 of a narrow round (measured: 20 us against 31 us at K = 5120) but holds an eighth of a narrow tile
     // each: it wins when the leftover is a few row tiles and the token count moderate (K=5120, N=17408, M=512: 256
     // wide tiles + 16 panels x 16 token blocks, 116.6 -> 102.4 us; at M=1024 the narrow tiles stay ahead).
-    static const int skinny_tail_on = getenv("RQ_GEMM_SKINNY_TAIL") ? atoi(getenv("RQ_GEMM_SKINNY_TAIL")) : 1;
     bool skinny_tail = false;
     // (the skinny kernel addresses the digit planes with 32-bit offsets)
     const bool planes_fit = (int64_t) a.L.ng * 128 * a.Mp < ((int64_t) 1 << 32);
-    if (skinny_tail_on && force < 0 && a.groups_per_fold == 1 && whole > 0 && whole < n_tiles && planes_fit) {
+    if (a.groups_per_fold == 1 && whole > 0 && whole < n_tiles && planes_fit) {
         const int tail_panels = a.L.n_panels - whole / n_tok_tiles * 4;
         const int64_t wgs = (int64_t) tail_panels * ((a.M + 31) / 32);
         const double c = 2.6 * (whole / kCUs) + 0.65 * ((wgs + kCUs - 1) / kCUs);
@@ -556,8 +553,7 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
         }
     }
     // the super-tile order of the wide kernel needs a wide region of whole blocks of 8 row tiles x 4 token tiles
-    static const int no_super = getenv("RQ_GEMM_SUPER") ? atoi(getenv("RQ_GEMM_SUPER")) == 0 : 0;
-    const int super_tiles = !no_super && n_wide > 0 && n_tok_tiles % 4 == 0 && n_wide % n_tok_tiles == 0 &&
+    const int super_tiles = n_wide > 0 && n_tok_tiles % 4 == 0 && n_wide % n_tok_tiles == 0 &&
                             (n_wide / n_tok_tiles) % 8 == 0;
     const uint4 *codes = reinterpret_cast<const uint4 *>(p + a.L.off_codes);
     const float *s_w = reinterpret_cast<const float *>(p + a.L.off_sw);

@@ -17,7 +17,6 @@
 // colsum_g is recomputed from the codes (dot8 against 0x11111111) instead of being stored.
 #include "rq_hadamard.h"
 
-#include <stdlib.h>
 
 #pragma clang fp contract(off)
 
@@ -308,18 +307,13 @@ hipError_t launch_twg(const GemvArgs &a, int nks, hipStream_t stream) {
 
 template <int T>
 hipError_t launch_t(const GemvArgs &a, int nks, hipStream_t stream) {
-    static const int waves = getenv("RQ_GEMV_WAVES") ? atoi(getenv("RQ_GEMV_WAVES")) : kGemvWaves;
     if constexpr (T <= kGemvWideTokens) {
         // activation groups of 128 / 256 (a format variant): one configuration
         if (a.gf == 2) return launch_twg<T, kGemvWaves, 2>(a, nks, stream);
         if (a.gf == 4) return launch_twg<T, kGemvWaves, 4>(a, nks, stream);
     }
     if (a.gf != 1) return hipErrorInvalidValue;
-    switch (waves) {
-        case 2:  return launch_twg<T, 2, 1>(a, nks, stream);
-        case 8:  return launch_twg<T, 8, 1>(a, nks, stream);
-        default: return launch_twg<T, 4, 1>(a, nks, stream);
-    }
+    return launch_twg<T, kGemvWaves, 1>(a, nks, stream);
 }
 
 }  // namespace
@@ -329,11 +323,8 @@ hipError_t launch_t(const GemvArgs &a, int nks, hipStream_t stream) {
 // about a thousand workgroups, at least a batch (kGemvWaves x kUnroll groups) each when K allows, at least ten groups
 // per workgroup, and never more than kMaxSlice (the slice's codes live in LDS).
 int gemv_ksplit(int n_panels, int ng) {
-    static const int forced = getenv("RQ_GEMV_KSPLIT") ? atoi(getenv("RQ_GEMV_KSPLIT")) : 0;
     int nks;
-    if (forced > 0) {
-        nks = forced;
-    } else {
+    {
         const int by_batch = (ng + kGemvWaves * kUnroll - 1) / (kGemvWaves * kUnroll);
         const int by_grid = (1024 + n_panels - 1) / n_panels;
         // more splits than ng / 10 cost more in atomics and short workgroups than they gain in parallelism (measured

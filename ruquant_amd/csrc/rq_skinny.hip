@@ -195,9 +195,9 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const uint8
     // workgroups of one panel's token blocks sit 8 apart in dispatch order: same XCD (ids go round-robin over the
     // eight XCDs), close in time
     const int bid = blockIdx.x;
-    const int chunk = nz == 1 ? bid >> 3 : nz == 2 ? bid >> 4 : bid / (8 * nz);
-    const int within = bid - chunk * 8 * nz;
-    const int unit = chunk * 8 + (within & 7), z = within >> 3;
+    const int chunk = nz == 1 ? bid / kXcds : nz == 2 ? bid / (2 * kXcds) : bid / (kXcds * nz);   // (shifts for 1 and 2)
+    const int within = bid - chunk * kXcds * nz;
+    const int unit = chunk * kXcds + within % kXcds, z = within / kXcds;
     if (unit >= n_units) return;
     const int t0 = z * kTok;                       // first token of this workgroup
     // Units of work: main_panels panels take their whole K in one workgroup (no atomics); each panel after them is
@@ -344,25 +344,14 @@ hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
 // the chip: `tail_split` slices per panel, which meet in 64-bit arrival cells. Device-scope atomics cost about 7 ns
 // per thousand, so the cut is chosen by a small cost model (busiest compute unit + atomics) rather than maximised.
 SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz) {
-    static const int forced = getenv("RQ_SKINNY_KSPLIT") ? atoi(getenv("RQ_SKINNY_KSPLIT")) : 0;
-    constexpr int kCUs = 256;
+    const int kCUs = device_compute_units();
     SkinnyPlan plan;
     const int smax = ng / 4 < 1 ? 1 : (ng / 4 > 16 ? 16 : ng / 4);   // at least four groups per slice
-    if (forced > 0) {
-        plan.main_panels = 0;
-        plan.tail_split = forced > smax ? smax : forced;
-        return plan;
-    }
     const int per_round = kCUs / nz;                       // panels in one round of the chip
     plan.main_panels = n_panels / per_round * per_round;
     plan.tail_split = 1;
     const int b = n_panels - plan.main_panels;
     if (b == 0) return plan;
-    static const int forced_tail = getenv("RQ_SKINNY_TAIL") ? atoi(getenv("RQ_SKINNY_TAIL")) : 0;
-    if (forced_tail > 0) {
-        plan.tail_split = forced_tail > smax ? smax : forced_tail;
-        return plan;
-    }
     // microseconds: a panel's weights at the rate one compute unit sustains, atomics at 7 ns per thousand (mostly
     // hidden behind the whole panels when there are any)
     const double t_panel = (double) ng * 2048.0 / (M <= 16 ? 19000.0 : 13000.0);
@@ -381,17 +370,16 @@ SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz) {
 }
 
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream) {
-    static const int tt1_max = getenv("RQ_SKINNY_TT1_MAX") ? atoi(getenv("RQ_SKINNY_TT1_MAX")) : 16;
+    constexpr int tt1_max = 16;   // most tokens served with one token tile of 16 per wavefront
     if (a.panels > 0) return launch_tt<2, false>(a, stream);   // the tail of a GEMM launch: blocks of 32 tokens
     if (a.mvals != nullptr) {   // the caller wrote single-plane activations
         // 33..64 tokens: one workgroup with four token tiles per wavefront reads the weights once and halves the
         // workgroup count, two blocks of 32 tokens give twice the workgroups. The former wins on long rows and on
         // weights with a whole round of panels (K=17408, N=5120, M=64: 22.7 against 26.9 us; K=5120, N=17408: 27.1
         // against 27.9), the latter on small weights (K=5120, N=5120: 10.9 against 15.8 us).
-        static const int wide_tokens = getenv("RQ_SKINNY_WIDE") ? atoi(getenv("RQ_SKINNY_WIDE")) : -1;
         int n_panels = 0;
         for (int i = 0; i < a.w.n; ++i) n_panels += a.w.L[i].n_panels;
-        const bool wide = wide_tokens >= 0 ? wide_tokens != 0 : (a.w.L[0].ng >= 160 || n_panels >= 256);
+        const bool wide = a.w.L[0].ng >= 160 || n_panels >= device_compute_units();
         if (a.M > 32 && wide) return launch_tt<4, true>(a, stream);
         if (a.M <= 16) return launch_tt<1, true>(a, stream);
         return launch_tt<2, true>(a, stream);
