@@ -71,6 +71,12 @@ int64_t rq_w4a4_tensor_rot(const void *host_block0, int type, int64_t K);
 /* Replaces ggml_rq_act_group (P:2623-2631): 64, or RQ_ACT_GROUP = 128 / 256 (read once). */
 int rq_w4a4_act_group(void);
 
+/* The weight-multiplier encoding of a tensor, from block 0's sum field (RQ_W_MULT / RQ_W_MULT_G, P:40-43): 0 = legacy
+ * row code sum (multiplier 1), 256 = one multiplier per block (1 << 30 | k), 64 = one per 64 inputs (3 << 29 | ...).
+ * Weight groups of 64 need activation groups of 64: ggml_vec_dot_w4a4_a4 asserts it (P:169-170), so a caller's first
+ * use refuses such a tensor when rq_w4a4_act_group() != 64 (the adapter aborts, the Python host raises). */
+int rq_w4a4_weight_group(const void *host_block0);
+
 /* ---- first use ------------------------------------------------------------------------------------ */
 
 /* Bytes of the prepared (streaming) form of an N x K weight; a multiple of 256. */
@@ -116,10 +122,15 @@ int rq_w4a4_mul_mat_static(int type, const void *prepared_dev, int64_t K, int64_
                            float *y_dev, int64_t ldy,
                            float clip, int64_t n_rot, rq_stream_t stream);
 
-/* Measurement aid with no counterpart in the reference: rq_w4a4_mul_mat split into its two stages so that the
- * product kernel can be timed alone. stages = 1: activation transform only (Hadamard + quantizer, also clears the
- * split-K scratch); 2: product + epilogue only, on the workspace a previous stages-1 call filled for the same
- * problem; 3: both (identical to rq_w4a4_mul_mat). */
+/* rq_w4a4_mul_mat in its two stages, for the reference's shared quantized activation (rq_act_cache, P:1996-2023,
+ * P:2160-2172): consecutive MUL_MATs of one x (q / k / v, gate / up) that were not fused rotate and quantize x once.
+ * stages = 1: activation transform only (Hadamard + quantizer; also clears the split-K cells of N rows);
+ * stages = 2: product + epilogue only, on a workspace that a stages-1 or stages-3 call filled for the same type, K, M,
+ *             x, clip and n_rot and for at least as many weight rows (cells of more rows were not cleared);
+ * stages = 3: both (identical to rq_w4a4_mul_mat). The workspace must have been zero-filled once when it was
+ * allocated if stage 2 is ever used on it with a different N than the filling call. One token on the one-launch
+ * decode path has no separate activation stage: stage 1 does nothing there and stage 2 is the whole operator.
+ * bench.py also uses the split to time the product kernel alone. */
 int rq_w4a4_mul_mat_stages(int type, const void *prepared_dev, int64_t K, int64_t N,
                            const float *x_dev, int64_t ldx, int64_t M,
                            float *y_dev, int64_t ldy,

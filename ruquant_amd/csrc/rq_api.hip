@@ -342,6 +342,15 @@ int rq_w4a4_hadamard_factor(int64_t n, int *p, int *m) {
 
 int rq_w4a4_act_group(void) { return env().act_group; }
 
+int rq_w4a4_weight_group(const void *host_block0) {
+    if (!host_block0) return 0;
+    uint32_t sum = 0;
+    memcpy(&sum, reinterpret_cast<const char *>(host_block0) + 4, sizeof sum);
+    if ((sum >> 29) == 3u) return 64;
+    if ((sum >> 30) == 1u) return 256;
+    return 0;
+}
+
 int rq_w4a4_supported(int type, int64_t K, int64_t N, int64_t M, int64_t ldx_bytes, int64_t ldy_bytes) {
     if (!shape_ok(type, K, N, M)) return 0;
     if (ldx_bytes % 16 != 0 || ldx_bytes < K * 4) return 0;

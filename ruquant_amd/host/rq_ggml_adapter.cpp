@@ -33,6 +33,44 @@ bool contiguous_blocks(const rq_tensor *t) {
     return t->nb[0] == RQ_BLOCK_BYTES && t->nb[1] == row;
 }
 
+bool capturing(rq_backend_context &ctx) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t) ctx.stream, &st) != hipSuccess) return false;
+    return st != hipStreamCaptureStatusNone;
+}
+
+// Makes the scratch buffer at least `bytes` long. Growing synchronizes, frees and allocates, none of which may happen
+// under graph capture: there the call aborts with a message instead (first_use sizes the buffer for max_tokens, so a
+// steady-state call gets here only with more tokens than the context was told to expect).
+void *scratch(rq_backend_context &ctx, size_t bytes) {
+    if (ctx.scratch_bytes < bytes) {
+        if (capturing(ctx)) {
+            rq_abort("scratch too small under graph capture: raise rq_backend_context::max_tokens", (long long) bytes,
+                     (long long) ctx.scratch_bytes);
+        }
+        hip_check(hipStreamSynchronize((hipStream_t) ctx.stream), "scratch");
+        if (ctx.scratch) hip_check(hipFree(ctx.scratch), "scratch");
+        hip_check(hipMalloc(&ctx.scratch, bytes), "scratch");
+        // the split-K cells inside must read zero before their first use (the kernels leave them zero)
+        hip_check(hipMemsetAsync(ctx.scratch, 0, bytes, (hipStream_t) ctx.stream), "scratch");
+        ctx.scratch_bytes = bytes;
+        ctx.act.valid = false;
+    }
+    return ctx.scratch;
+}
+
+// largest workspace any token count up to max_tokens needs for this weight
+size_t workspace_for(int type, int64_t K, int64_t N, int64_t max_tokens) {
+    size_t need = 0;
+    const int64_t probes[] = { 1, 3, 4, 8, 9, 16, 17, 64, 65, max_tokens };
+    for (int64_t m : probes) {
+        if (m > max_tokens) continue;
+        const size_t b = rq_w4a4_workspace_bytes(type, K, N, m);
+        if (b > need) need = b;
+    }
+    return need;
+}
+
 // first use, never inside a graph capture: read block 0's header, resolve clip and rotation length, prepare
 rq_first_use *first_use(rq_backend_context &ctx, const rq_tensor *src0) {
     if (src0->extra) return (rq_first_use *) src0->extra;
@@ -49,21 +87,16 @@ rq_first_use *first_use(rq_backend_context &ctx, const rq_tensor *src0) {
     }
     fu->prepared_bytes = rq_w4a4_prepared_bytes(src0->ne[0], src0->ne[1]);
     hip_check(hipMalloc(&fu->prepared, fu->prepared_bytes), "prepared weight");
+    if (rq_w4a4_weight_group(&hdr) == 64 && rq_w4a4_act_group() != 64) {
+        // ggml_vec_dot_w4a4_a4 asserts the same (P:169-170): one weight multiplier per activation group
+        rq_abort("weight groups of 64 need activation groups of 64 (RQ_ACT_GROUP)", rq_w4a4_act_group());
+    }
     const int rc = rq_w4a4_prepare(src0->data, src0->ne[0], src0->ne[1], fu->prepared, fu->prepared_bytes, ctx.stream);
     if (rc != 0) rq_abort("rq_w4a4_prepare failed", rc);
+    // the workspace of every later call with up to max_tokens tokens: allocated now, outside capture
+    scratch(ctx, workspace_for(src0->type, src0->ne[0], src0->ne[1], ctx.max_tokens));
     const_cast<rq_tensor *>(src0)->extra = fu;
     return fu;
-}
-
-void *scratch(rq_backend_context &ctx, size_t bytes) {
-    if (ctx.scratch_bytes < bytes) {
-        // growing is a first-use event too: let the stream drain before the old buffer goes away
-        hip_check(hipStreamSynchronize((hipStream_t) ctx.stream), "scratch");
-        if (ctx.scratch) hip_check(hipFree(ctx.scratch), "scratch");
-        hip_check(hipMalloc(&ctx.scratch, bytes), "scratch");
-        ctx.scratch_bytes = bytes;
-    }
-    return ctx.scratch;
 }
 
 }  // namespace
@@ -111,11 +144,39 @@ void ggml_cuda_mul_mat_rq_w4a4_fused(rq_backend_context &ctx, const rq_tensor *c
         Nws = 0;
         for (int i = 0; i < n; ++i) Nws += (Ns[i] + 63) / 64 * 64;
     }
-    const size_t ws_bytes = rq_w4a4_workspace_bytes(src0s[0]->type, K, Nws, M);
+    size_t ws_bytes = rq_w4a4_workspace_bytes(src0s[0]->type, K, Nws, M);
+    if (ws_bytes > ctx.scratch_bytes && n > 1 && capturing(ctx)) {
+        // a fused set that was not sized for: cells for the largest weight are enough (one product launch per weight)
+        ws_bytes = rq_w4a4_workspace_bytes(src0s[0]->type, K, Nmax, M);
+        Nws = Nmax;
+    }
     void *ws = scratch(ctx, ws_bytes);
-    const int rc = rq_w4a4_mul_mat_fused(src0s[0]->type, n, prepared, K, Ns, (const float *) src1->data,
-                                         (int64_t) (src1->nb[1] / sizeof(float)), M, ys, ldys, fu0->clip, fu0->n_rot, ws,
-                                         ws_bytes, ctx.stream);
+    const int type = src0s[0]->type;
+    const float *x = (const float *) src1->data;
+    const int64_t ldx = (int64_t) (src1->nb[1] / sizeof(float));
+    rq_act_cache &c = ctx.act;
+    int rc;
+    if (n == 1 && c.valid && c.src1 == src1 && c.data == src1->data && c.type == type && c.clip == fu0->clip &&
+        c.n_rot == fu0->n_rot && c.K == K && c.M == M && (Ns[0] + 63) / 64 * 64 <= c.rows_cleared) {
+        // the scratch still holds this x rotated and quantized: the product alone (reference: P:2167-2172)
+        ++ctx.act_hits;
+        rc = rq_w4a4_mul_mat_stages(type, prepared[0], K, Ns[0], x, ldx, M, ys[0], ldys[0], fu0->clip, fu0->n_rot, ws,
+                                    ctx.scratch_bytes, ctx.stream, 2);
+    } else {
+        ++ctx.act_misses;
+        rc = rq_w4a4_mul_mat_fused(type, n, prepared, K, Ns, x, ldx, M, ys, ldys, fu0->clip, fu0->n_rot, ws, ws_bytes,
+                                   ctx.stream);
+        c.src1 = src1;
+        c.data = src1->data;
+        c.type = type;
+        c.clip = fu0->clip;
+        c.n_rot = fu0->n_rot;
+        c.K = K;
+        c.M = M;
+        // (a fused call may have cleared the cells of all its weights; the largest one is what it surely cleared)
+        c.rows_cleared = (Nmax + 63) / 64 * 64;
+        c.valid = rc == 0;
+    }
     if (rc != 0) rq_abort("no path for this shape", rc);   // the reference: GGML_ABORT (P:2337)
 }
 
@@ -136,4 +197,12 @@ bool ggml_cuda_rq_w4a4_can_fuse(const rq_tensor *a, const rq_tensor *b) {
     return ia != nullptr && ib != nullptr && ia->clip == ib->clip && ia->n_rot == ib->n_rot;
 }
 
-void ggml_cuda_rq_graph_begin(rq_backend_context &ctx) { (void) ctx; }
+void ggml_cuda_rq_graph_begin(rq_backend_context &ctx) { ctx.act.valid = false; }
+
+void ggml_cuda_rq_w4a4_release(rq_tensor *src0) {
+    rq_first_use *fu = (rq_first_use *) src0->extra;
+    if (!fu) return;
+    (void) hipFree(fu->prepared);
+    delete fu;
+    src0->extra = nullptr;
+}

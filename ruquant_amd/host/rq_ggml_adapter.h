@@ -22,13 +22,31 @@ struct rq_tensor {
     rq_tensor *src[2];
 };
 
+// The quantized activation the scratch buffer currently holds (the reference's rq_act_cache, P:1996-2023): consecutive
+// MUL_MATs of one x (q / k / v, gate / up) that were not fused still share one rotation + quantization. Keyed like
+// the reference's (P:2163-2166) on the src1 tensor, its data pointer, the type and the weight-side parameters; dropped
+// at every graph evaluation (ggml_cuda_rq_graph_begin), because x may have changed in place since.
+struct rq_act_cache {
+    const void *src1 = nullptr, *data = nullptr;
+    int         type = 0;
+    float       clip = 0.0f;
+    int64_t     n_rot = 0, K = 0, M = 0;
+    int64_t     rows_cleared = 0;   // split-K cells of this many weight rows were cleared when the activation was made
+    bool        valid = false;
+};
+
 // Stands in for ggml_backend_cuda_context: the stream every launch goes to and a scratch pool. The pool here is
-// one growing device buffer owned by the context (ggml's is stream ordered; the op only needs "memory that stays
-// valid until the stream has passed this call").
+// one device buffer owned by the context (ggml's is stream ordered; the op only needs "memory that stays valid until
+// the stream has passed this call"). It is sized at a weight's first use, which is outside graph capture, for every
+// token count up to max_tokens (the backend's micro-batch), so that steady-state calls never allocate; a call that
+// needs more grows it when the stream is not capturing and aborts with a message when it is.
 struct rq_backend_context {
-    void  *stream = nullptr;
-    void  *scratch = nullptr;
-    size_t scratch_bytes = 0;
+    void        *stream = nullptr;
+    void        *scratch = nullptr;
+    size_t       scratch_bytes = 0;
+    int64_t      max_tokens = 512;
+    rq_act_cache act;
+    long long    act_hits = 0, act_misses = 0;
     ~rq_backend_context();
 };
 
@@ -45,6 +63,8 @@ bool ggml_cuda_rq_w4a4_can_fuse(const rq_tensor *a, const rq_tensor *b);
 // n <= 3 such products as one call (reference: P:2371-2380)
 void ggml_cuda_mul_mat_rq_w4a4_fused(rq_backend_context &ctx, const rq_tensor *const *src0s, rq_tensor *const *dsts, int n,
                                      const rq_tensor *src1);
-// starts a new graph evaluation (reference: P:2021-2023). This implementation keeps no cross-call activation cache,
-// so there is nothing to drop.
+// starts a new graph evaluation (reference: P:2021-2023): drops the shared quantized activation
 void ggml_cuda_rq_graph_begin(rq_backend_context &ctx);
+// frees what a weight's first use allocated (the reference never frees its rq_tensor_info; a backend that unloads
+// models calls this from its buffer-free path)
+void ggml_cuda_rq_w4a4_release(rq_tensor *src0);

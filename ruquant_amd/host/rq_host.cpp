@@ -5,7 +5,10 @@
 //
 // weights.bin: N rows of K/256 blocks (144 bytes each) as a W4A4 / W4A4H tensor stores them; x.bin: M x K floats;
 // y.bin (written): M x N floats. With three extra arguments "fuse <weights2.bin> <N2> <y2.bin>" a second weight of
-// the same x goes through ggml_cuda_rq_w4a4_can_fuse / _fused.
+// the same x goes through ggml_cuda_rq_w4a4_can_fuse / _fused. With "cache <weights2.bin> <N2> <y2.bin>" the two
+// weights run as separate calls inside one graph evaluation (the second reuses the first's quantized activation),
+// then x is negated in place and a new evaluation runs both again: y.bin / y2.bin hold the results for -x, and
+// <y2.bin>.first the second weight's result of the first evaluation; the JSON carries the hit / miss counts.
 #include "rq_ggml_adapter.h"
 
 #include <hip/hip_runtime.h>
@@ -69,7 +72,8 @@ int main(int argc, char **argv) {
     int iters = 20;
     int argi = 8;
     if (argc > argi && strcmp(argv[argi], "fuse") != 0) iters = atoi(argv[argi++]);
-    const bool fuse = argc > argi + 3 && strcmp(argv[argi], "fuse") == 0;
+    const bool cache = argc > argi + 3 && strcmp(argv[argi], "cache") == 0;
+    const bool fuse = argc > argi + 3 && (strcmp(argv[argi], "fuse") == 0 || cache);
     const int64_t N2 = fuse ? atoll(argv[argi + 2]) : 0;
 
     int n_dev = 0;
@@ -130,12 +134,44 @@ int main(int argc, char **argv) {
     CK(hipStreamSynchronize(stream));
     const bool ready_after = ggml_cuda_rq_w4a4_ready(&w);
 
+    long long hits_first = 0, misses_first = 0, hits_again = 0, misses_again = 0;
+    if (cache) {
+        // one graph evaluation, two separate calls of the same x: the second finds x already rotated and quantized
+        ctx.act_hits = ctx.act_misses = 0;
+        ggml_cuda_rq_graph_begin(ctx);
+        ggml_cuda_mul_mat_rq_w4a4(ctx, &w, &x, &y);
+        ggml_cuda_mul_mat_rq_w4a4(ctx, &w2, &x, &y2);
+        CK(hipStreamSynchronize(stream));
+        hits_first = ctx.act_hits;
+        misses_first = ctx.act_misses;
+        {
+            std::vector<float> y2h((size_t) M * N2);
+            CK(hipMemcpy(y2h.data(), y2d, y2h.size() * 4, hipMemcpyDeviceToHost));
+            const std::string first = std::string(argv[argi + 3]) + ".first";
+            FILE *ff = fopen(first.c_str(), "wb");
+            if (!ff || fwrite(y2h.data(), 4, y2h.size(), ff) != y2h.size()) return 1;
+            fclose(ff);
+        }
+        // x changes in place between evaluations: the new evaluation must not reuse the old activation
+        float *xf = reinterpret_cast<float *>(xh.data());
+        for (size_t i = 0; i < (size_t) M * K; ++i) xf[i] = -xf[i];
+        CK(hipMemcpy(xd, xh.data(), x_bytes, hipMemcpyHostToDevice));
+        ctx.act_hits = ctx.act_misses = 0;
+        ggml_cuda_rq_graph_begin(ctx);
+        ggml_cuda_mul_mat_rq_w4a4(ctx, &w, &x, &y);
+        ggml_cuda_mul_mat_rq_w4a4(ctx, &w2, &x, &y2);
+        CK(hipStreamSynchronize(stream));
+        hits_again = ctx.act_hits;
+        misses_again = ctx.act_misses;
+        iters = 0;
+    }
+
     // steady state
     std::vector<double> times;
     for (int i = 0; i < iters; ++i) {
         const auto t0 = std::chrono::steady_clock::now();
         ggml_cuda_rq_graph_begin(ctx);
-        if (fuse && ggml_cuda_rq_w4a4_can_fuse(&y, &y2)) {
+        if (fuse && !cache && ggml_cuda_rq_w4a4_can_fuse(&y, &y2)) {
             const rq_tensor *ws[2] = { &w, &w2 };
             rq_tensor *ds[2] = { &y, &y2 };
             ggml_cuda_mul_mat_rq_w4a4_fused(ctx, ws, ds, 2, &x);
@@ -163,9 +199,10 @@ int main(int argc, char **argv) {
         fclose(f);
     }
     printf("{\"supported\": true, \"device\": \"%s\", \"type\": %d, \"K\": %lld, \"N\": %lld, \"M\": %lld, "
-           "\"ready_before\": %s, \"ready_after\": %s, \"fused\": %s, \"iters\": %d, \"best_us\": %.2f, \"mean_us\": %.2f}\n",
+           "\"ready_before\": %s, \"ready_after\": %s, \"fused\": %s, \"iters\": %d, \"best_us\": %.2f, \"mean_us\": %.2f, "
+           "\"act_hits_first\": %lld, \"act_misses_first\": %lld, \"act_hits_again\": %lld, \"act_misses_again\": %lld}\n",
            prop.name, type, (long long) K, (long long) N, (long long) M, ready_before ? "true" : "false",
            ready_after ? "true" : "false", fused_ran ? "true" : "false", iters, iters ? best : 0.0,
-           iters ? sum / iters : 0.0);
+           iters ? sum / iters : 0.0, hits_first, misses_first, hits_again, misses_again);
     return 0;
 }

@@ -33,6 +33,7 @@ PROTOTYPES = {
     "rq_w4a4_resolve_clip": (ctypes.c_float, [ctypes.c_void_p, ctypes.c_int]),
     "rq_w4a4_tensor_rot": (ctypes.c_int64, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64]),
     "rq_w4a4_act_group": (ctypes.c_int, []),
+    "rq_w4a4_weight_group": (ctypes.c_int, [ctypes.c_void_p]),
     "rq_w4a4_prepared_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64]),
     "rq_w4a4_prepare": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
                                        ctypes.c_size_t, ctypes.c_void_p]),

@@ -84,6 +84,10 @@ class W4A4Weight:
         if self.type == TYPE_W4A4H and self.n_rot < 0:
             raise RqError("W4A4H: Hadamard length %d does not divide this row of %d"
                           % (int(blocks[0, 0]["pad"][0]), self.K))
+        b0 = np.ascontiguousarray(blocks[0, 0]).view(np.uint8)
+        if L.rq_w4a4_weight_group(b0.ctypes.data) == 64 and L.rq_w4a4_act_group() != 64:
+            # the reference asserts the same in ggml_vec_dot_w4a4_a4 (patch lines 169-170)
+            raise RqError("weight groups of 64 need activation groups of 64 (RQ_ACT_GROUP=%d)" % L.rq_w4a4_act_group())
         raw = torch.from_numpy(blocks.view(np.uint8).reshape(-1).copy()).to(self.device)
         nbytes = L.rq_w4a4_prepared_bytes(self.K, self.N)
         if nbytes == 0:

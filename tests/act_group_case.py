@@ -23,6 +23,15 @@ cases = [(rq.TYPE_W4A4H, 200, 1536, 0), (rq.TYPE_W4A4H, 200, 1536, 64), (rq.TYPE
          (rq.TYPE_W4A4H, 256, 5120, 0), (rq.TYPE_W4A4H, 320, 768, 64), (rq.TYPE_W4A4H, 128, 17408, 0)]
 for type_, N, K, wgroup in cases:
     blocks, wf = adversarial_weights(rq_oracle, N, K, type_, wgroup=wgroup)
+    if wgroup == 64:
+        # weight groups of 64 need activation groups of 64: the reference asserts (patch lines 169-170), this refuses
+        try:
+            rq.W4A4Weight(blocks, type_, DEV)
+            print("wgroup=64 with RQ_ACT_GROUP=%d was not refused" % G, flush=True)
+            bad += 1
+        except rq.RqError as e:
+            print("wgroup=64 refused: %s" % e, flush=True)
+        continue
     W = rq.W4A4Weight(blocks, type_, DEV)
     for M in (1, 2, 3, 5, 8, 9, 40, 130):   # up to eight tokens: the GEMV folds the wide groups; beyond: the narrow-tile GEMM
         x = adversarial_activations(M, K, type_, wf, seed=M)
@@ -32,6 +41,25 @@ for type_, N, K, wgroup in cases:
         print("mul_mat type=%d N=%d K=%d wgroup=%d M=%d: %s" % (type_, N, K, wgroup, M,
                                                                 "ok" if ok else first_mismatch(got, want)), flush=True)
         bad += not ok
+# the reference's own shape list (test-backend-ops, patch lines 3024-3040), both types
+from test_gpu_parity import _shapes_reference  # noqa: E402
+last = None
+for N, M, K in sorted(_shapes_reference(), key=lambda s: (s[0], s[2], s[1])):
+    for type_ in (rq.TYPE_W4A4, rq.TYPE_W4A4H):
+        if K % G != 0:
+            continue
+        if last is None or last[0] != (N, K, type_):
+            blocks, wf = adversarial_weights(rq_oracle, N, K, type_)
+            last = ((N, K, type_), blocks, wf, rq.W4A4Weight(blocks, type_, DEV))
+        _, blocks, wf, W = last
+        x = adversarial_activations(M, K, type_, wf, seed=M)
+        got = run_gpu(W, x)
+        want = rq_oracle.mul_mat(type_, blocks, x, W.clip, n_rot=max(W.n_rot, 0), G=G)
+        ok = bits_equal(got, want)
+        if not ok:
+            print("reference shape type=%d N=%d M=%d K=%d: %s" % (type_, N, M, K, first_mismatch(got, want)), flush=True)
+        bad += not ok
+print("reference shapes done", flush=True)
 for K, had in ((1536, True), (5120, True), (1024, False)):
     rng = np.random.default_rng(K)
     x = (rng.standard_normal((3, K)) * np.exp2(rng.integers(-3, 4, size=(3, K // 64)).repeat(64, axis=1))).astype(np.float32)

@@ -62,6 +62,30 @@ def test_host_fuses_two_weights_of_one_input(oracle, tmp_path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("M", [2, 16, 70])
+def test_host_shares_the_quantized_activation_between_separate_calls(oracle, tmp_path, M):
+    """Two MUL_MATs of one x as separate calls inside one graph evaluation (the reference's rq_act_cache, patch lines
+    2160-2172): the second is a hit and still bit-identical; after x changed in place and a new evaluation began, the
+    first call is a miss again and both results are those of the new x."""
+    type_, K, N, N2 = rq.TYPE_W4A4H, 5120, 640, 256
+    b1 = synth.random_weight_blocks(N, K, 41, type_, clip=0.9)
+    b2 = synth.random_weight_blocks(N2, K, 42, type_, clip=0.9)
+    x = synth.activations("outlier_channels", M, K, 43)
+    b2.tofile(tmp_path / "w2.bin")
+    r, y = _run(tmp_path, type_, K, N, M, b1, x, extra=("cache", tmp_path / "w2.bin", N2, tmp_path / "y2.bin"))
+    assert r.returncode == 0, r.stderr
+    info = json.loads(r.stdout.strip().splitlines()[-1])
+    assert (info["act_hits_first"], info["act_misses_first"]) == (1, 1)
+    assert (info["act_hits_again"], info["act_misses_again"]) == (1, 1)
+    c = float(np.float32(0.9))
+    y2_first = np.fromfile(str(tmp_path / "y2.bin") + ".first", dtype=np.float32).reshape(M, N2)
+    assert bits_equal(y2_first, oracle.mul_mat(type_, b2, x, c, n_rot=K)), "hit differs from a fresh transform"
+    y2 = np.fromfile(tmp_path / "y2.bin", dtype=np.float32).reshape(M, N2)
+    assert bits_equal(y, oracle.mul_mat(type_, b1, -x, c, n_rot=K)), "stale activation after graph_begin"
+    assert bits_equal(y2, oracle.mul_mat(type_, b2, -x, c, n_rot=K))
+
+
+@pytest.mark.gpu
 def test_host_reports_unsupported_shape(tmp_path):
     # K with no Hadamard factorization: the backend declines, ggml would fall back to the CPU
     type_, K, N, M = rq.TYPE_W4A4H, 7 * 256, 64, 1
