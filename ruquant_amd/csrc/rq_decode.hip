@@ -107,11 +107,11 @@ __device__ __forceinline__ void rot_sync(int *cnt, int &target, int lane) {
     wait_count<false>(cnt, target);
 }
 
-// LDS: [row][row (Paley output)][g_lo][g_hi][codes][mz][cells][wave maxima, unit]
+// LDS: [row, padded][Paley output, dense][codes][mz][cells][wave maxima, unit, phase counter]
 __host__ __device__ inline size_t decode_lds_bytes(int K, bool two_rows) {
     const int Kp = ((K + (K >> 4) + 1) + 3) & ~3;
     const int ng = K / kGroup;
-    return (size_t) ((two_rows ? 2 : 1) * Kp + 2 * ng + K / 8 + ng + kDecodeCells + 8 + kRotWaves + 4) * 4;
+    return (size_t) (Kp + (two_rows ? K : 0) + K / 8 + ng + kDecodeCells + 8 + kRotWaves + 4) * 4;
 }
 
 // MG: group-items (64 rows x one group: two loads) a stream wavefront has in flight per round of a whole panel;
@@ -126,10 +126,8 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
     const int K = a.K, ng = K / kGroup;
     const int Kp = align4(padi(K) + 1);
     float *buf = smem;
-    float *alt = smem + Kp;
-    float *g_lo = smem + (P > 1 ? 2 : 1) * Kp;
-    float *g_hi = g_lo + ng;
-    uint32_t *s_act = reinterpret_cast<uint32_t *>(g_hi + ng);     // [K / 8] code words, tensor nibble order
+    float *alt = smem + Kp;   // Paley output, dense (its readers take 8 consecutive floats as two 16-byte reads)
+    uint32_t *s_act = reinterpret_cast<uint32_t *>(smem + Kp + (P > 1 ? K : 0));   // [K / 8] code words, tensor nibble order
     int32_t *s_mz = reinterpret_cast<int32_t *>(s_act + K / 8);    // [ng] m | (8 - z) << 8
     int32_t *red = s_mz + ng;                                      // cells: [whole panels][64 rows], [octets][8 rows], one spare
     float *s_part = reinterpret_cast<float *>(red + kDecodeCells + 8);   // [kRotWaves] widest range per wavefront
@@ -451,41 +449,38 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                 // Paley across the P chunks of every rotation block, into the second row buffer. A wave-item is
                 // (slice of kOut outputs, run of 64 columns); the slice's sign pattern is straight-line code.
                 constexpr int kOut = P / 4;
+                constexpr int kSlices = 4;
                 const int ncols = K / P;
                 const int pm = m + (m >> 4);
                 const int col_runs = (ncols + 63) >> 6;
-                const int n_it = 4 * col_runs;
+                const int n_it = kSlices * col_runs;
                 const int per_wave = (n_it + kRotWaves - 1) / kRotWaves;
                 for (int it = 0; it < per_wave; ++it) {
                     const int wi = wave * per_wave + it;
                     if (wi >= n_it) break;
-                    const int s = (wi >= col_runs) + (wi >= 2 * col_runs) + (wi >= 3 * col_runs);   // wi / col_runs
-                    const int cidx = (wi - s * col_runs) * 64 + lane;
+                    int s = 0, cr = wi;   // wi / col_runs, wi % col_runs (a few uniform subtractions)
+                    while (cr >= col_runs) {
+                        cr -= col_runs;
+                        ++s;
+                    }
+                    const int cidx = cr * 64 + lane;
                     if (cidx >= ncols) continue;
                     const int rb = cidx >> lm, j = cidx & (m - 1);   // chunk lengths are powers of two
                     const int b0 = rb * a.n_rot + j;
-                    float col[P];
                     const float *src = buf + padi(b0);
                     float out[kOut];
                     if (m == 256) {
-                        // chunks of 256: the chunk stride in the padded row is the constant 272, so the P loads and the
-                        // kOut stores are immediate offsets from one address
-#pragma unroll
-                        for (int i = 0; i < P; ++i) col[i] = src[i * 272];
-                        paley_pick<P, kOut>(s, col, out);
-                        float *dst = alt + padi(b0) + kOut * s * 272;
-#pragma unroll
-                        for (int o = 0; o < kOut; ++o) dst[o * 272] = out[o] * a.scale;
+                        // chunks of 256: the chunk stride in the padded row is the constant 272, so the P loads are
+                        // immediate offsets from one address
+                        paley_pick_stream<P, kOut, 272>(s, src, 272, out);
                     } else {
-#pragma unroll
-                        for (int i = 0; i < P; ++i) col[i] = src[i * pm];
-                        paley_pick<P, kOut>(s, col, out);
-#pragma unroll
-                        for (int o = 0; o < kOut; ++o) alt[padi(b0 + (kOut * s + o) * m)] = out[o] * a.scale;
+                        paley_pick_stream<P, kOut, 0>(s, src, pm, out);
                     }
+                    float *dst = alt + b0 + kOut * s * m;
+#pragma unroll
+                    for (int o = 0; o < kOut; ++o) dst[o * m] = out[o] * a.scale;
                 }
                 rot_sync(s_cnt, sync_target, lane);
-                buf = alt;
             } else {
                 for (int i = rt; i < K; i += kRotThreads) buf[padi(i)] = buf[padi(i)] * a.scale;
                 rot_sync(s_cnt, sync_target, lane);
@@ -497,6 +492,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         // a thread per code word, eight lanes per group of 64; the word's eight values stay in registers for the codes
         const int nw = K >> 3;
         constexpr int kWordRounds = 4;   // K <= 16384
+        const bool dense = a.rotate && P > 1;            // the Paley stage wrote the dense buffer
         float f[kWordRounds][8];
         float g_lo_r[kWordRounds], g_hi_r[kWordRounds];
         float rmax = 0.0f;
@@ -505,9 +501,20 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
             const int w = wr * kRotThreads + rt;
             if (wr * kRotThreads < nw) {   // uniform
                 const bool on = w < nw;
-                const float *sp = buf + padi(8 * (on ? w : 0));
+                if (dense) {
+                    const float4 *sp = reinterpret_cast<const float4 *>(alt + 8 * (on ? w : 0));
+                    const float4 v0 = sp[0], v1 = sp[1];
+                    f[wr][0] = v0.x; f[wr][1] = v0.y; f[wr][2] = v0.z; f[wr][3] = v0.w;
+                    f[wr][4] = v1.x; f[wr][5] = v1.y; f[wr][6] = v1.z; f[wr][7] = v1.w;
+                } else {
+                    const float *sp = buf + padi(8 * (on ? w : 0));
 #pragma unroll
-                for (int j = 0; j < 8; ++j) f[wr][j] = on ? sp[j] : 0.0f;
+                    for (int j = 0; j < 8; ++j) f[wr][j] = sp[j];
+                }
+                if (!on) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) f[wr][j] = 0.0f;
+                }
                 float mn = fminf(fminf(fminf(fminf(0.0f, f[wr][0]), fminf(f[wr][1], f[wr][2])),
                                        fminf(fminf(f[wr][3], f[wr][4]), fminf(f[wr][5], f[wr][6]))), f[wr][7]);
                 float mx = fmaxf(fmaxf(fmaxf(fmaxf(0.0f, f[wr][0]), fmaxf(f[wr][1], f[wr][2])),
@@ -578,7 +585,13 @@ hipError_t launch_pmt(const DecodeKernelArgs &k, int grid, size_t lds, hipStream
 // items per wavefront and round beside whole panels, 12 when the launch is remainder only
 template <int P>
 hipError_t launch_p(const DecodeKernelArgs &k, int grid, size_t lds, hipStream_t stream) {
-    if (k.main_panels == 0) return launch_pmt<P, 0, 12>(k, grid, lds, stream);
+    if (k.main_panels == 0) {
+        // remainder only: all of a wavefront's items in flight when they are at most 26
+        const int octets = (k.q_base + 2) / 2 + 1;
+        const int per_wave = (octets * (k.K / 256) + kStrWaves - 1) / kStrWaves;
+        if (per_wave > 12) return launch_pmt<P, 0, 26>(k, grid, lds, stream);
+        return launch_pmt<P, 0, 12>(k, grid, lds, stream);
+    }
     const int gpw = (k.K / kGroup + kStrWaves - 1) / kStrWaves;
     const bool tail = k.q_base > 0 || k.q_extra > 0;
     if (gpw % 12 == 0 || (gpw % 10 != 0 && gpw > 10)) {
@@ -596,6 +609,7 @@ hipError_t allow_lds() {
 template <int P>
 hipError_t allow_lds_p() {
     hipError_t e = allow_lds<P, 0, 12>();
+    if (e == hipSuccess) e = allow_lds<P, 0, 26>();
     if (e == hipSuccess) e = allow_lds<P, 10, 4>();
     if (e == hipSuccess) e = allow_lds<P, 10, 0>();
     if (e == hipSuccess) e = allow_lds<P, 12, 2>();
@@ -618,6 +632,9 @@ bool decode_takes(int K, int rotate, int p, int m, int act_group) {
     if (act_group != kGroup) return false;
     if (K > 16384) return false;
     if (rotate) {
+        // Long Paley stages stay with the rotation kernel that spreads a token over many workgroups: H68 x H256
+        // (K = 17408) is 1.2 M additions per token, which one workgroup's eight wavefronts need 14 us for (measured:
+        // 28 us for the whole call against 17.5 us with the two launches).
         if (p != 1 && p != 12 && p != 20) return false;
         if ((m & 15) != 0) return false;
     }

@@ -72,6 +72,26 @@ __device__ __forceinline__ void paley_pick(int s, const float (&col)[P], float (
     }
 }
 
+// The same outputs with the column read on the fly (element i of the column at src[i * stride]): the loop runs over
+// the column's elements and updates the O running sums, so every sum still receives its terms in ascending chunk
+// order, one rounding per term, and a long column needs O + 1 registers instead of P.
+template <int P, int O, int STRIDE, int S = 0>
+__device__ __forceinline__ void paley_pick_stream(int s, const float *src, int stride, float (&out)[O]) {
+    if (s == S) {
+        constexpr PaleyTable<P> T = make_paley<P>();
+#pragma unroll
+        for (int o = 0; o < O; ++o) out[o] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < P; ++i) {
+            const float c = src[i * (STRIDE ? STRIDE : stride)];
+#pragma unroll
+            for (int o = 0; o < O; ++o) out[o] = T.neg[i][O * S + o] ? out[o] - c : out[o] + c;
+        }
+    } else if constexpr (S + 1 < P / O) {
+        paley_pick_stream<P, O, STRIDE, S + 1>(s, src, stride, out);
+    }
+}
+
 // all P outputs of one column, written back in place (the column is private to the calling thread). STRIDE is the
 // distance between the chunks of a column in the padded row when it is known at compile time (0: use `stride`): the
 // P loads and P stores then share one or two address registers with immediate offsets, where a run-time stride costs
