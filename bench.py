@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA
 # HBM bytes per launch of the headline's dominant kernel come from the committed rocprofv3 counter summary (FETCH_SIZE
 # and WRITE_SIZE passes, each scaled by a plain copy of known size): the line "traffic_bytes_per_launch: <n>" in it
-HEADLINE_PROFILE = os.path.join(ROOT, "profiles", "gemv_m1_k5120_n17408.md")
+HEADLINE_PROFILE = os.path.join(ROOT, "profiles", "decode_m1_k5120_n17408.md")
 
 
 def profiled_traffic_bytes(path=HEADLINE_PROFILE):
@@ -164,6 +164,7 @@ class Layer:
                                   [rq.fused_workspace_bytes([w["q"], w["k"], w["v"]], M),
                                    rq.fused_workspace_bytes([w["gate"], w["up"]], M)]),
                               dtype=torch.uint8, device=dev)
+        self.shared = rq.SharedActivation(self.ws)
         self.code_bytes = sum(K * N // 2 for _, K, N in self.SHAPES)
         self.bytes = sum(algorithmic_bytes(K, N, M) for _, K, N in self.SHAPES)
         self.ops = sum(2 * M * K * N for _, K, N in self.SHAPES)
@@ -173,6 +174,15 @@ class Layer:
         w = self.sets[self.i % len(self.sets)]
         self.i += 1
         rq, o = self.rq, self.out
+        if fused == "shared":
+            # seven separate calls, but q / k / v and gate / up share one rotation + quantization of their x (the
+            # reference's activation cache)
+            sa = self.shared
+            sa.begin()
+            for n, src in (("q", self.x0), ("k", self.x0), ("v", self.x0), ("o", o["q"]), ("gate", o["o"]),
+                           ("up", o["o"]), ("down", o["up"])):
+                sa.mul_mat(w[n], src, o[n])
+            return
         if fused:
             rq.mul_mat_fused([w["q"], w["k"], w["v"]], self.x0, outs=[o["q"], o["k"], o["v"]], workspace=self.ws)
         else:
@@ -210,11 +220,13 @@ class Layer:
     def measure(self, steps, warmup):
         fused_ms = self.timed(steps, warmup, True)
         plain_ms = self.timed(steps, warmup, False)
+        shared_ms = self.timed(steps, warmup, "shared")
         return {"M": self.M, "matmuls": 7, "code_bytes": self.code_bytes, "layer_us": round(fused_ms * 1e3, 2),
                 "layer_gbs": round(self.bytes / fused_ms / 1e6, 1),
                 "layer_frac_of_hbm_peak": round(self.bytes / fused_ms / 1e6 / HBM_PEAK_GBS, 4),
                 "layer_tops": round(self.ops / fused_ms / 1e9, 2),
-                "layer_us_seven_separate_calls": round(plain_ms * 1e3, 2)}
+                "layer_us_seven_separate_calls": round(plain_ms * 1e3, 2),
+                "layer_us_seven_calls_shared_activation": round(shared_ms * 1e3, 2)}
 
 
 def host_cores():
@@ -460,7 +472,11 @@ def main():
                    "algorithmic_bytes": b},
         "roofline": {"bound": "hbm", "achieved": round(b / kern_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(b / kern_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": profiled_traffic_bytes(),
-                     "kernel": "rq_gemv_kernel<1, 4, 1>", "kernel_us": round(kern_ms * 1e3, 3)},
+                     # one token: rotation, quantizer, product and epilogue are ONE launch, so the dominant kernel
+                     # is the whole operator (template arguments: Paley order, groups and remainder items in flight)
+                     "kernel": "rq_decode_kernel<20, 10, 4>" if res["activation_kernel_us"] < 1.0
+                               else "rq_gemv_kernel<1, 4, 1>",
+                     "kernel_us": round(kern_ms * 1e3, 3)},
         "roofline_m2048": roofline_m2048,
         "cpu_baseline": cpu,
         "parity_vs_oracle": parity,

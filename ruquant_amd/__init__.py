@@ -8,6 +8,6 @@ from .lib import load_library, build_library, LibraryMissing  # noqa: F401
 from .w4a4 import (  # noqa: F401
     TYPE_W4A4, TYPE_W4A4H, TYPE_A4, TYPE_A4H, BLOCK_DTYPE,
     W4A4Weight, supported, hadamard_factor, resolve_clip, tensor_rot,
-    mul_mat, mul_mat_fused, fused_workspace_bytes, hadamard, quantize_act, RqError,
+    mul_mat, mul_mat_fused, fused_workspace_bytes, hadamard, quantize_act, RqError, SharedActivation,
     pack, pack_groups, set_clip, set_rot_len, dequantize_rows, quantize_weights, dequantize,
 )

@@ -188,12 +188,10 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         const int32_t f1 = __builtin_nontemporal_load(a.ws.flags[1]);
         const int32_t f2 = __builtin_nontemporal_load(a.ws.flags[2]);
 
-        // Behind this barrier the rotate wavefronts have the row. Not one weight is requested before: with 2 (4) of a
-        // wavefront's 22 loads ahead of the barrier the row arrived later and the whole call took 12.0 (12.5) us
-        // instead of 11.2.
         // Behind this barrier the rotate wavefronts have the row. Not one weight is requested before: with 1, 2, 4
         // or 9 of a wavefront's 10 groups ahead of the barrier the row arrives later and the whole call takes 11.9,
-        // 11.7, 12.5 and 15.3 us instead of 11.0.
+        // 11.7, 12.5 and 15.3 us instead of 11.0; even a single 4-byte read per wavefront (to have the weight pages
+        // translated early) costs 0.5 us, because a wavefront's loads return in order and that first one is slow.
         __builtin_amdgcn_s_barrier();
         RQ_STAMP(1);
 
@@ -204,11 +202,12 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         bool waited = false;
 
         // remainder item `i` of this workgroup -> address of its 1 KiB (8 rows x 4 groups x 2 halves)
-        // (items past the end read the first KiB of the remainder again: valid memory whatever this workgroup owns)
+        // (items past the end read the workgroup's own first KiB again, so that those reads spread over the memory
+        // channels like the real ones; a workgroup without remainder rows takes the remainder's first KiB: valid memory)
         auto tail_address = [&](int i, bool valid) -> const uint8_t * {
-            const int ol = (int) (((uint32_t) i * (uint32_t) a.inv_nblk) >> 22);
+            const int ol = valid ? (int) (((uint32_t) i * (uint32_t) a.inv_nblk) >> 22) : 0;
             const int bb = valid ? i - ol * nblk : 0;
-            const int o = valid ? oct0 + ol : a.tail_panel0 * 8;
+            const int o = n_items > 0 ? oct0 + ol : a.tail_panel0 * 8;
             const int panel = o >> 3;
             const int wsel = (panel >= a.ws.first[1]) + (panel >= a.ws.first[2]);
             const int wpanel = panel - (wsel == 0 ? 0 : wsel == 1 ? a.ws.first[1] : a.ws.first[2]);
@@ -587,7 +586,7 @@ template <int P>
 hipError_t launch_p(const DecodeKernelArgs &k, int grid, size_t lds, hipStream_t stream) {
     if (k.main_panels == 0) {
         // remainder only: all of a wavefront's items in flight when they are at most 26
-        const int octets = (k.q_base + 2) / 2 + 1;
+        const int octets = (k.q_base + (k.q_extra > 0 ? 1 : 0) + 1) / 2 + 1;   // most octets a run of quads touches
         const int per_wave = (octets * (k.K / 256) + kStrWaves - 1) / kStrWaves;
         if (per_wave > 12) return launch_pmt<P, 0, 26>(k, grid, lds, stream);
         return launch_pmt<P, 0, 12>(k, grid, lds, stream);

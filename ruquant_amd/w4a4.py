@@ -146,6 +146,43 @@ def mul_mat_fused(weights, x, outs=None, workspace=None, clip=None):
     return outs
 
 
+class SharedActivation:
+    """The reference's rq_act_cache (patch lines 1996-2023, 2160-2172) for this host: consecutive MUL_MATs of one x
+    that were not fused rotate and quantize x once. The cache is the workspace itself; `begin()` plays
+    ggml_cuda_rq_graph_begin (x may have changed in place since the last evaluation)."""
+
+    def __init__(self, workspace):
+        self.workspace = workspace
+        workspace.zero_()            # the split-K cells inside must read zero before stage 2 first uses them
+        self.key = None
+        self.rows_cleared = 0
+        self.hits = self.misses = 0
+
+    def begin(self):
+        self.key = None
+
+    def mul_mat(self, weight, x, out):
+        L = load_library()
+        M, K = x.shape
+        key = (x.data_ptr(), x.stride(0), M, K, weight.type, weight.clip, weight.n_rot)
+        rows = (weight.N + 63) // 64 * 64
+        hit = key == self.key and rows <= self.rows_cleared
+        ldx = x.stride(0) if M > 1 else K
+        ldy = out.stride(0) if M > 1 else weight.N
+        with torch.cuda.device(x.device):
+            rc = L.rq_w4a4_mul_mat_stages(weight.type, weight.prepared.data_ptr(), K, weight.N, x.data_ptr(), ldx, M,
+                                          out.data_ptr(), ldy, weight.clip, max(weight.n_rot, 0),
+                                          self.workspace.data_ptr(), self.workspace.numel(), _stream_ptr(),
+                                          2 if hit else 3)
+        _check(rc, "rq_w4a4_mul_mat_stages")
+        if hit:
+            self.hits += 1
+        else:
+            self.misses += 1
+            self.key, self.rows_cleared = key, rows
+        return out
+
+
 def hadamard(x, n_rot=None):
     """x[M, K] -> x diag(H, H, ...) with H of length n_rot (default K), as ggml_rq_hadamard does per block."""
     L = load_library()
