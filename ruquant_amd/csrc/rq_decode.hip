@@ -124,6 +124,31 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
     RQ_STAMP_DECL;
     RQ_STAMP(0);
     const int K = a.K, ng = K / kGroup;
+
+    // ---- the rotate wavefronts request the row before anything else: 16 consecutive floats per thread and unit.
+    // Everything below (cells, row scales, item addresses) is computed while it travels.
+    // Chunks of 256 floats (16 units): the 16 lanes of a DPP row hold one chunk, so the Sylvester stages with
+    // strides 16 .. 128 run between lanes and the row makes no trip through LDS between its stages. Lane l of a row
+    // holds the unit whose index bits (b0, b1, b2, b3) give l = b0 ^ 2 b1 ^ 7 b2 ^ 8 b3: the partners of the four
+    // stages are then l ^ 1, l ^ 2, l ^ 7, l ^ 8, which are single DPP controls.
+    const bool dpp256 = a.rotate && a.m == 256;
+    const int lr = lane & 15;
+    const int hb3 = lr >> 3, hr = lr & 7, hb2 = hr >> 2, hr2 = hr ^ (hb2 ? 7 : 0);
+    const int unit_of_lane = (hr2 & 1) | (hr2 & 2) | hb2 << 2 | hb3 << 3;
+    constexpr int kUnits = 2;   // K <= 16384
+    float4 qv[kUnits][4];
+    if (wave < kRotWaves) {
+#pragma unroll
+        for (int ub = 0; ub < kUnits; ++ub) {
+            int u = tid + ub * kRotThreads;
+            if (dpp256) u = (u & ~15) | unit_of_lane;
+            if (u < (K >> 4)) {
+                const float4 *src = reinterpret_cast<const float4 *>(a.x + 16 * u);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) qv[ub][j] = src[j];
+            }
+        }
+    }
     const int Kp = align4(padi(K) + 1);
     float *buf = smem;
     float *alt = smem + Kp;   // Paley output, dense (its readers take 8 consecutive floats as two 16-byte reads)
@@ -322,7 +347,8 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                 for (int it = 0; it < MT; ++it) {
                     const int iq = i0 + sw + it * kStrWaves;
                     const bool on = iq < n_items;
-                    const int i = on ? iq : 0;
+                    if (!on) break;   // (uniform over the wavefront; the items behind are past the end as well)
+                    const int i = iq;
                     const int ol = (int) (((uint32_t) i * (uint32_t) a.inv_nblk) >> 22);
                     const int bb = i - ol * nblk;
                     const int g = 4 * bb + g4;
@@ -355,8 +381,8 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                     }
                     term >>= kTermShift;
                     // rows of a shared octet that belong to the neighbour land in cells that nobody writes out; items
-                    // past the end go to the spare cell
-                    if (h == 0) atomicAdd(&red[on ? main_cells + ol * 8 + r8 : kDecodeCells], term);
+                    // past the end add nothing (a shared spare cell for them made all their lanes queue on one address)
+                    if (h == 0 && on) atomicAdd(&red[main_cells + ol * 8 + r8], term);
                 }
             }
         }
@@ -367,27 +393,6 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         // =========================================================== the activation side (512 threads)
         const int rt = tid;
         int sync_target = 0;
-        // the row, 16 consecutive floats per thread and unit; all loads go out before the first barrier.
-        // Chunks of 256 floats (16 units): the 16 lanes of a DPP row hold one chunk, so the Sylvester stages with
-        // strides 16 .. 128 run between lanes and the row makes no trip through LDS between its stages. Lane l of a row
-        // holds the unit whose index bits (b0, b1, b2, b3) give l = b0 ^ 2 b1 ^ 7 b2 ^ 8 b3: the partners of the four
-        // stages are then l ^ 1, l ^ 2, l ^ 7, l ^ 8, which are single DPP controls.
-        const bool dpp256 = a.rotate && a.m == 256;
-        const int lr = lane & 15;
-        const int hb3 = lr >> 3, hr = lr & 7, hb2 = hr >> 2, hr2 = hr ^ (hb2 ? 7 : 0);
-        const int unit_of_lane = (hr2 & 1) | (hr2 & 2) | hb2 << 2 | hb3 << 3;
-        constexpr int kUnits = 2;   // K <= 16384
-        float4 qv[kUnits][4];
-#pragma unroll
-        for (int ub = 0; ub < kUnits; ++ub) {
-            int u = rt + ub * kRotThreads;
-            if (dpp256) u = (u & ~15) | unit_of_lane;
-            if (u < (K >> 4)) {
-                const float4 *src = reinterpret_cast<const float4 *>(a.x + 16 * u);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) qv[ub][j] = src[j];
-            }
-        }
         // The stream starts only when the row has ARRIVED: requests queued behind the weight stream are served
         // after it (a row requested just before the stream took 5 us instead of 1.5).
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
