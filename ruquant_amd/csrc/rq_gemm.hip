@@ -8,8 +8,11 @@
 // lo in [-32, 31] and hi in [-60, 60]. Then
 //     m_g S_g = 64 Xhi_g + Xlo_g,   floor(m_g S_g / 16) = 4 Xhi_g + floor(Xlo_g / 16),
 // where Xhi_g = sum w hi accumulates ACROSS groups inside the MFMA accumulator (no vector work at all) and only
-// Xlo_g = sum w lo needs the per-group floor: one arithmetic shift and one add per output and group, both
-// full-rate ops. Two MFMAs per group instead of one, but the vector ALU no longer paces the loop.
+// Xlo_g = sum w lo needs the per-group floor. That floor rides on the accumulator too: the low-digit accumulator
+// holds 256 h + r (h = floors so far, r = the last group's remainder); clearing r with one AND per output and
+// group and handing the result to the next group's MFMA as its C operand yields Xlo' + 256 h, whose floor by 256
+// is floor(Xlo' / 256) + h (Xlo' = 16 Xlo, see below). Two MFMAs per group instead of one, and one full-rate
+// vector instruction per output and group.
 //
 // Weight codes stay packed (int4) all the way into LDS and are widened when a wavefront reads its A fragment, by
 // masking each nibble into the HIGH half of a byte (w * 16, no sign extension needed), so every X above arrives
@@ -184,10 +187,8 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint
     }
 }
 
-// Two groups of a wide tile at once (the fast path: no weight multipliers). With both groups' low-digit sums at
-// hand the fold is lo += (Sa >> 8) + (Sb >> 8): two shifts and ONE three-operand add, a quarter fewer vector
-// instructions than group by group. Software pipeline in units of one 16 x 16 tile (x two groups = 4 MFMAs): the
-// MFMAs of unit i are issued while the vector ALU folds unit i - 1.
+// Two groups of a tile at once (the fast path: no weight multipliers), in units of one 16 x 16 tile (x two groups =
+// 4 MFMAs); the second group of a unit is issued one unit later, when the first group's result has arrived.
 template <bool NARROW>
 __device__ __forceinline__ void compute_pair(const Ctx &c, const Stage &sa, const Stage &sb,
                                              v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
@@ -208,7 +209,12 @@ __device__ __forceinline__ void compute_pair(const Ctx &c, const Stage &sa, cons
         widen(pb.y, e1, o1);
         Ab[rt] = v4i{ e0, o0, e1, o1 };
     }
-    v4i Sa[2], Sb[2];
+    // lo[rt][ct] is a chained accumulator here: value = 256 h + r, h = the sum of the floors so far, 0 <= r < 256.
+    // Clearing r (one AND per value) and feeding the result to the next group's low-digit MFMA as its C operand gives
+    // X + 256 h, whose floor by 256 is floor(X / 256) + h: the MFMA adds the floors up, and the vector ALU spends one
+    // instruction per value and group instead of a shift and half a three-operand add. The kernel shifts once at the end.
+    auto cleared = [](const v4i &v) { return v4i{ v[0] & ~255, v[1] & ~255, v[2] & ~255, v[3] & ~255 }; };
+    v4i T[2];      // after group a, per unit in flight
     v4i B[2][4];   // [buffer][lo a, hi a, lo b, hi b] of one token tile; the next tile's are fetched a unit ahead
     auto load_b = [&](int buf, int ct) {
         B[buf][0] = as_v4i(sa.cell[b_off + 16 * ct]);
@@ -221,25 +227,20 @@ __device__ __forceinline__ void compute_pair(const Ctx &c, const Stage &sa, cons
     for (int un = 0; un < 4 * TT + 1; ++un) {
         const int ct = un >> 2, rt = un & 3;
         if (rt == 0) __builtin_amdgcn_sched_barrier(0);   // keeps the LDS reads of later tiles from piling up early
+        if (un > 0) {
+            // group b of the previous unit: its group-a result has had a unit's worth of MFMAs to arrive. (Before the
+            // next tile's B fragments are fetched: they go into the buffer that unit 4 ct - 1 still reads.)
+            const int pct = (un - 1) >> 2, prt = (un - 1) & 3;
+            const v4i r = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ab[prt], B[pct & 1][2], cleared(T[(un - 1) & 1]), 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) lo[prt][pct][i] = r[i];
+            hi[prt][pct] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ab[prt], B[pct & 1][3], hi[prt][pct], 0, 0, 0);
+        }
         if (un < 4 * TT) {
             if (rt == 0 && ct < TT - 1) load_b((ct + 1) & 1, ct + 1);
-            Sa[un & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aa[rt], B[ct & 1][0], v4i{ 0, 0, 0, 0 }, 0, 0, 0);
-            Sb[un & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ab[rt], B[ct & 1][2], v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+            const v4i cur = v4i{ lo[rt][ct][0], lo[rt][ct][1], lo[rt][ct][2], lo[rt][ct][3] };
+            T[un & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aa[rt], B[ct & 1][0], cleared(cur), 0, 0, 0);
             hi[rt][ct] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Aa[rt], B[ct & 1][1], hi[rt][ct], 0, 0, 0);
-            hi[rt][ct] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ab[rt], B[ct & 1][3], hi[rt][ct], 0, 0, 0);
-        }
-        if (un > 0) {
-            const int pct = (un - 1) >> 2, prt = (un - 1) & 3;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) lo[prt][pct][i] += (Sa[(un - 1) & 1][i] >> 8) + (Sb[(un - 1) & 1][i] >> 8);
-        }
-        if (un > 0 && un < 4 * TT) {
-            // 4 MFMAs interleaved with the 12 vector ops of the previous unit's fold
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-                __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);  // VALU
-            }
         }
     }
 }
@@ -445,13 +446,15 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
         gemm_body<false, NARROW>(c, s0, s1, s2, s3, s4, s5, k_src, hi, lo);
     }
 
+    // (the fast path leaves the sum of the floors in the bits above the low byte: see compute_pair)
+    const bool chained = !(flags[0] & 1) && !(NARROW && c.gs > 1);
     int32_t tot[4][TT][4];
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
 #pragma unroll
         for (int ct = 0; ct < TT; ++ct) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) tot[rt][ct][i] = (hi[rt][ct][i] >> 2) + lo[rt][ct][i];
+            for (int i = 0; i < 4; ++i) tot[rt][ct][i] = (hi[rt][ct][i] >> 2) + (chained ? lo[rt][ct][i] >> 8 : lo[rt][ct][i]);
         }
     }
     if (NARROW) {
