@@ -213,6 +213,7 @@ __device__ __forceinline__ void compute_pair(const Ctx &c, const Stage &sa, cons
     // Clearing r (one AND per value) and feeding the result to the next group's low-digit MFMA as its C operand gives
     // X + 256 h, whose floor by 256 is floor(X / 256) + h: the MFMA adds the floors up, and the vector ALU spends one
     // instruction per value and group instead of a shift and half a three-operand add. The kernel shifts once at the end.
+    // (|X| <= 16 x 64 x 8 x 32 = 2^18 per group, so |256 h| < 2^18 x K / 64 <= 2^27 for the longest row: no overflow.)
     auto cleared = [](const v4i &v) { return v4i{ v[0] & ~255, v[1] & ~255, v[2] & ~255, v[3] & ~255 }; };
     v4i T[2];      // after group a, per unit in flight
     v4i B[2][4];   // [buffer][lo a, hi a, lo b, hi b] of one token tile; the next tile's are fetched a unit ahead

@@ -167,6 +167,42 @@ def test_mul_mat_longest_row(oracle, type_, M):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
+def test_gemm_wide_tiles_longest_row_extreme_sums(oracle):
+    """K = 32768 on the wide tiles of the MFMA GEMM with inputs that drive the integer sums to their ends: rows whose
+    codes are all -8 or all +7 against tokens that quantize to q - z = +15 or -15 with m = 255 in every one of the
+    512 groups (a token of equal positive values: lo = 0, z = 0, every q clamps to 15; of equal negative values:
+    z = 15, q = 0). The low-digit accumulator then carries 512 floors of magnitude 480 above its low byte, the
+    high-digit accumulator 512 x 491520. 16 row tiles x 12 token tiles = 192 tiles: the launch plan runs them wide
+    (one round of wide tiles is cheaper than three rounds of narrow ones). Checked on a sample of tokens (tokens are
+    independent: the oracle gets the sampled rows of x)."""
+    N, K, M, type_ = 4096, 32768, 1536, rq.TYPE_W4A4
+    blocks = synth.random_weight_blocks(N, K, 5, type_, clip=0.9)
+    qs = blocks["qs"].reshape(N, -1)
+    qs[0, :] = 0x88888888
+    qs[1, :] = 0x77777777
+    qs[2, ::2] = 0x88888888
+    qs[2, 1::2] = 0x77777777
+    blocks["qs"] = qs.reshape(blocks["qs"].shape)
+    blocks["sum"] = synth.signed_code_sums(qs).astype(np.int32)[:, None]
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    x = synth.activations("outlier_channels", M, K, 9)
+    x[0, :] = 1.0
+    x[1, :] = -1.0
+    x[2, :] = np.where((np.arange(K) // 64) % 2 == 0, 1.0, -1.0)
+    x[3, :] = np.where(np.arange(K) % 2 == 0, 3.0, -3.0)
+    x[1535, :] = 0.5
+    got = run_gpu(W, x)
+    sample = [0, 1, 2, 3, 4, 127, 128, 700, 1534, 1535]
+    want = oracle.mul_mat(type_, blocks, x[sample], W.clip, n_rot=0)
+    assert bits_equal(got[sample], want), first_mismatch(got[sample], want)
+    # closed form of the first extreme, independent of the oracle: every group contributes floor(255 x (-8 x 15 x 64)
+    # / 16) = -122400, the token's unit is (1.0 x clip) / 3825
+    clip = np.float32(0.9)
+    unit = np.float32(np.float32(1.0) * clip) / np.float32(3825.0)
+    expect = (np.float32(-122400 * 512) * np.float32(16.0)) * unit * blocks["d"][0, 0]
+    assert got[0, 0] == np.float32(expect)
+
+
 def test_mul_mat_block_diagonal_rotation(oracle):
     """Hadamard length shorter than the row (pad[0] = K / 4), as ruquant convert --rot-blocks writes."""
     N, K, M, type_ = 128, 6144, 9, rq.TYPE_W4A4H
