@@ -156,10 +156,10 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     if (ws_bytes < W.bytes || (reinterpret_cast<uintptr_t>(ws) & 255) != 0) return RQ_E_WORKSPACE;
     uint8_t *wsb = reinterpret_cast<uint8_t *>(ws);
 
-    // Activation groups of 128 / 256 (RQ_ACT_GROUP) change where the per-group floor falls. The GEMV folds at that
-    // granularity for up to kGemvWideTokens tokens (one token 16 us, eight 33 us at K = 5120, N = 17408); beyond
-    // that only the narrow-tile MFMA kernel does (44 us from 4 to 64 tokens), so every larger token count takes it
-    // (a format variant, not a tuned path).
+    // Activation groups of 128 / 256 (RQ_ACT_GROUP) change where the per-group floor falls. The GEMV and the skinny
+    // kernel (single-plane form) fold at that granularity over the same token ranges as with groups of 64 (K = 5120,
+    // N = 17408, groups of 128: four tokens 19.6 us on the GEMV, nine 18.3 us on the skinny kernel); beyond 64 tokens
+    // the narrow-tile MFMA kernel does (a format variant, not a tuned path).
     const int G = env().act_group;
     if (M == 1 && env().decode_fused && decode_takes((int) K, type == RQ_TYPE_W4A4H, p, m, G)) {
         // one token: rotation, quantizer, product and epilogue in one launch, all weights of a fused call included
@@ -184,7 +184,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
         d.compute_units = device_compute_units();
         return (int) launch_decode(d, stream);
     }
-    const Path path = G != 64 ? (M <= kGemvWideTokens ? kPathGemv : kPathGemm) : path_of(M);
+    const Path path = path_of(M);
     const bool gemm = path != kPathGemv;   // the int8 digit planes feed both MFMA kernels
     RotQuantArgs q;
     memset(&q, 0, sizeof q);
@@ -203,7 +203,8 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     // microseconds, so the rotation runs spread over workgroups (ranges out) and a second small kernel quantizes.
     // (up to 40 tokens: from there on the one-workgroup-per-token kernel has enough tokens to fill the chip: K = 17408,
     // 64 tokens: 17.9 us against 21.2 us)
-    const bool two_step = path == kPathSkinny && q.rotate && p >= 44 && (m & 63) == 0 && M <= kTwoStepTokens;
+    // (the second kernel reads ranges per run of 64: activation groups of 64 only)
+    const bool two_step = path == kPathSkinny && G == kGroup && q.rotate && p >= 44 && (m & 63) == 0 && M <= kTwoStepTokens;
     q.mode = gemm && !two_step ? kActI8 : kActStats;
     q.u = reinterpret_cast<float *>(wsb + W.off_u);
     q.act = reinterpret_cast<uint32_t *>(wsb + W.off_i8);
@@ -270,6 +271,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             g.u = q.u;
             g.M = (int) M;
             g.Mp = act_mp;
+            g.runs_per_group = G / kGroup;
             g.tot = reinterpret_cast<int32_t *>(wsb + W.off_tot);
             g.panel0 = 0;
             g.panels = 0;

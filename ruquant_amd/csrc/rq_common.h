@@ -235,6 +235,7 @@ struct SkinnyArgs {
     const uint8_t  *mvals;  // null: two digit planes
     const float    *u;      // [Mp]
     int             M, Mp;
+    int             runs_per_group;   // runs of 64 per activation group: 1, or 2 / 4 with RQ_ACT_GROUP = 128 / 256 (single plane only)
     int32_t        *tot;    // split-K cells [M][panels of all weights * 64], 64 bits each
     // a sub-range of the (single) weight's panels, whole K per workgroup, any number of 32-token blocks: the tail of
     // a GEMM launch (rq_gemm.hip). panels == 0: all panels, planned by skinny_plan.
@@ -245,7 +246,7 @@ struct SkinnyPlan {
     int main_panels;   // leading panels that run as one whole-K workgroup each
     int tail_split;    // K slices (workgroups) per remaining panel
 };
-SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz);
+SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz, int runs_per_group = 1);
 
 // One token, one launch (rq_decode.hip): every workgroup rotates and quantizes the token for itself behind its share of
 // the weight stream; rows are dealt in quads, whole K per workgroup, so no sums cross workgroups.

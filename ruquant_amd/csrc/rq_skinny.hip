@@ -136,25 +136,86 @@ __device__ __forceinline__ void mma_frag(const Frag<TT, SINGLE> &f, const uint8_
     }
 }
 
-// One wavefront's share of the K slice: groups g_first, g_first + kWaves, ... (n of them). Ring slot j % D holds
-// group j; the slot is refilled with group j + D as soon as group j's MFMAs have been issued. The scheduling
-// barriers keep the compiler from sinking those loads to their first use (which would expose the whole memory
-// latency once per group). Past the end the ring issues idle loads, and nothing consumes them.
-template <int TT, bool SINGLE>
-__device__ __forceinline__ void fill_ring(Frag<TT, SINGLE> (&ring)[depth_of(TT)], const uint8_t *a_panel, uint32_t a_lane,
-                                          const uint8_t *b_planes, uint32_t b_lane, const uint8_t *mvals,
-                                          uint32_t m_lane, int Mp, int g_first, int n) {
+// Activation groups of 128 / 256 (RQ_ACT_GROUP), single plane: the quantizer's multiplier, and with it the floor of
+// the fold, covers gf = 2 or 4 consecutive runs of 64 (reference patch lines 160-170). The runs' sums chain through
+// the MFMA accumulator (`acc`) and are folded once, at the group's last run, with the weight multiplier of its first
+// run, as the reference takes it. `g` is the run's index in the row, so g % gf is its place in the group (uniform).
+// |16 sum| < 2^19 and k m < 2^12: the 24-bit multiply and its 32-bit result are exact.
+template <int TT, bool HASK>
+__device__ __forceinline__ void mma_frag_wide(const Frag<TT, true> &f, const uint8_t *k_base, int g, int gf,
+                                              v4i (&acc)[4][TT], int32_t (&lo)[4][TT][4]) {
+    v4i A[4];
 #pragma unroll
-    for (int i = 0; i < depth_of(TT); ++i) {
-        load_frag<TT, SINGLE>(ring[i], a_panel, a_lane, b_planes, b_lane, mvals, m_lane, g_first + i * kWaves, Mp, i < n);
+    for (int rt = 0; rt < 4; ++rt) {
+        int e0, o0, e1, o1;
+        widen(f.a[rt].x, e0, o0);
+        widen(f.a[rt].y, e1, o1);
+        A[rt] = v4i{ e0, o0, e1, o1 };
+    }
+    const int pos = g & (gf - 1);
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+        const v4i B = v4i{ (int) f.b[tt][0].x, (int) f.b[tt][0].y, (int) f.b[tt][0].z, (int) f.b[tt][0].w };
+        if (pos == 0) {
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) acc[rt][tt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], B, v4i{ 0, 0, 0, 0 }, 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) acc[rt][tt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[rt], B, acc[rt][tt], 0, 0, 0);
+        }
+    }
+    if (pos != gf - 1) return;
+    int kk[4][4];
+    if (HASK) {
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+            const uint32_t k4 = *reinterpret_cast<const uint32_t *>(k_base + (size_t) (g - pos) * kPanelRows + 16 * rt);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) kk[rt][i] = (k4 >> (8 * i)) & 0xFF;
+        }
+    }
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+        const int mg = (int) f.mv[tt];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) lo[rt][tt][i] += __mul24(acc[rt][tt][i], HASK ? kk[rt][i] * mg : mg) >> 8;
+        }
     }
 }
 
-template <int TT, bool HASK, bool SINGLE>
+// One wavefront's share of the K slice: activation groups u_first, u_first + kWaves, ... of gf = 1 << gsh runs each
+// (n runs in all; gf = 1: the runs g_first, g_first + kWaves, ...). Ring slot j % D holds
+// the wavefront's run j; the slot is refilled with group j + D as soon as group j's MFMAs have been issued. The scheduling
+// barriers keep the compiler from sinking those loads to their first use (which would expose the whole memory
+// latency once per group). Past the end the ring issues idle loads, and nothing consumes them.
+__device__ __forceinline__ int run_at(int u_first, int gsh, int j) {
+    return ((u_first + (j >> gsh) * kWaves) << gsh) + (j & ((1 << gsh) - 1));
+}
+
+template <int TT, bool SINGLE>
+__device__ __forceinline__ void fill_ring(Frag<TT, SINGLE> (&ring)[depth_of(TT)], const uint8_t *a_panel, uint32_t a_lane,
+                                          const uint8_t *b_planes, uint32_t b_lane, const uint8_t *mvals,
+                                          uint32_t m_lane, int Mp, int u_first, int gsh, int n) {
+#pragma unroll
+    for (int i = 0; i < depth_of(TT); ++i) {
+        load_frag<TT, SINGLE>(ring[i], a_panel, a_lane, b_planes, b_lane, mvals, m_lane, run_at(u_first, gsh, i), Mp, i < n);
+    }
+}
+
+template <int TT, bool HASK, bool SINGLE, bool WIDE>
 __device__ __forceinline__ void stream_slice(Frag<TT, SINGLE> (&ring)[depth_of(TT)], const uint8_t *a_panel,
                                              uint32_t a_lane, const uint8_t *b_planes, uint32_t b_lane,
                                              const uint8_t *mvals, uint32_t m_lane, const uint8_t *k_base, int Mp,
-                                             int g_first, int n, v4i (&hi)[4][TT], int32_t (&lo)[4][TT][4]) {
+                                             int u_first, int gsh, int n, v4i (&hi)[4][TT], int32_t (&lo)[4][TT][4]) {
+    auto mma = [&](const Frag<TT, SINGLE> &f, int g) __attribute__((always_inline)) {
+        if constexpr (WIDE) {
+            mma_frag_wide<TT, HASK>(f, k_base, g, 1 << gsh, hi, lo);
+        } else {
+            mma_frag<TT, HASK, SINGLE>(f, k_base, g, hi, lo);
+        }
+    };
     constexpr int D = depth_of(TT);
     // whole rounds of the ring: branch-free, so the wait counts before each group's MFMAs are exact
     const int rounds = n / D;
@@ -162,11 +223,10 @@ __device__ __forceinline__ void stream_slice(Frag<TT, SINGLE> (&ring)[depth_of(T
 #pragma unroll
         for (int i = 0; i < D; ++i) {
             const int j = r * D + i;
-            const int g = g_first + j * kWaves;
             __builtin_amdgcn_sched_barrier(0);
-            mma_frag<TT, HASK, SINGLE>(ring[i], k_base, g, hi, lo);
+            mma(ring[i], run_at(u_first, gsh, j));
             __builtin_amdgcn_sched_barrier(0);
-            load_frag<TT, SINGLE>(ring[i], a_panel, a_lane, b_planes, b_lane, mvals, m_lane, g + D * kWaves, Mp, j + D < n);
+            load_frag<TT, SINGLE>(ring[i], a_panel, a_lane, b_planes, b_lane, mvals, m_lane, run_at(u_first, gsh, j + D), Mp, j + D < n);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -174,14 +234,15 @@ __device__ __forceinline__ void stream_slice(Frag<TT, SINGLE> (&ring)[depth_of(T
     const int rem = n - rounds * D;
 #pragma unroll
     for (int i = 0; i < D - 1; ++i) {
-        if (i < rem) mma_frag<TT, HASK, SINGLE>(ring[i], k_base, g_first + (rounds * D + i) * kWaves, hi, lo);
+        if (i < rem) mma(ring[i], run_at(u_first, gsh, rounds * D + i));
     }
 }
 
-template <int TT, bool SINGLE>
+// WIDE: activation groups of gf = 1 << gsh runs of 64 (single plane only); slices of K are then counted in groups.
+template <int TT, bool SINGLE, bool WIDE = false>
 __global__ void __launch_bounds__(kThreads, TT == 1 ? 4 : (SINGLE && TT == 2) ? 3 : 2)   // wavefronts per SIMD: 4 = two workgroups per CU
 rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const uint8_t *__restrict__ mvals,
-                 const float *__restrict__ u, int M, int Mp,
+                 const float *__restrict__ u, int M, int Mp, int gsh,
                  int n_units, int nz,
                  unsigned long long *__restrict__ cells, int n_rows_pad, int main_panels, int tail_split,
                  int slice_base, int slice_extra, int panel0) {
@@ -207,7 +268,8 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const uint8
     // filling up.
     const int ng = ws.ng;
     const int tail_units = n_units - main_panels;
-    int panel = unit - tail_units, ks = 0, nks = 1, g_begin = 0, g_end = ng;
+    // (g_begin, g_end: in activation groups, i.e. runs of 64 unless WIDE)
+    int panel = unit - tail_units, ks = 0, nks = 1, g_begin = 0, g_end = WIDE ? ng >> gsh : ng;
     if (unit < tail_units) {
         const int q = unit / tail_split;
         panel = main_panels + q;
@@ -263,18 +325,19 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const uint8
 
     // the first loads go out before anything that waits (the LDS clear)
     const int g_first = g_begin + wave;
-    const int n = g_first < g_end ? (g_end - g_first + kWaves - 1) / kWaves : 0;
+    const int gs = WIDE ? gsh : 0;
+    const int n = g_first < g_end ? ((g_end - g_first + kWaves - 1) / kWaves) << gs : 0;   // runs of this wavefront
     Frag<TT, SINGLE> ring[depth_of(TT)];
-    fill_ring<TT, SINGLE>(ring, a_panel, a_lane, b_planes, b_lane, mvals, m_lane, Mp, g_first, n);
+    fill_ring<TT, SINGLE>(ring, a_panel, a_lane, b_planes, b_lane, mvals, m_lane, Mp, g_first, gs, n);
     __builtin_amdgcn_sched_barrier(0);
 
     for (int i = tid; i < 64 * kStride; i += kThreads) s_tot[i] = 0;
 
     if (n > 0) {
         if (has_k) {
-            stream_slice<TT, true, SINGLE>(ring, a_panel, a_lane, b_planes, b_lane, mvals, m_lane, k_base, Mp, g_first, n, hi, lo);
+            stream_slice<TT, true, SINGLE, WIDE>(ring, a_panel, a_lane, b_planes, b_lane, mvals, m_lane, k_base, Mp, g_first, gs, n, hi, lo);
         } else {
-            stream_slice<TT, false, SINGLE>(ring, a_panel, a_lane, b_planes, b_lane, mvals, m_lane, k_base, Mp, g_first, n, hi, lo);
+            stream_slice<TT, false, SINGLE, WIDE>(ring, a_panel, a_lane, b_planes, b_lane, mvals, m_lane, k_base, Mp, g_first, gs, n, hi, lo);
         }
     }
 
@@ -313,24 +376,26 @@ rq_skinny_kernel(const WeightSet ws, const uint4 *__restrict__ act8, const uint8
     }
 }
 
-template <int TT, bool SINGLE>
+template <int TT, bool SINGLE, bool WIDE = false>
 hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
     const WeightSet ws = make_weight_set(a.w);
     const int n_panels = a.panels > 0 ? a.panels : ws.first[kMaxFused];
     const int nz = (a.M + TT * 16 - 1) / (TT * 16);
+    const int gf = WIDE ? a.runs_per_group : 1, gsh = gf == 4 ? 2 : gf == 2 ? 1 : 0;
+    const int n_groups = ws.ng / gf;   // what a slice of K is counted in
     SkinnyPlan plan;
     if (a.panels > 0) {   // whole K per workgroup: no arrival cells
         plan.main_panels = n_panels;
         plan.tail_split = 1;
     } else {
-        plan = skinny_plan(n_panels, ws.ng, a.M, nz);
+        plan = skinny_plan(n_panels, ws.ng, a.M, nz, gf);
     }
     const int n_units = plan.main_panels + (n_panels - plan.main_panels) * plan.tail_split;
     const int blocks = (n_units + 7) / 8 * 8 * nz;
-    hipLaunchKernelGGL((rq_skinny_kernel<TT, SINGLE>), dim3(blocks), dim3(kThreads), 0, stream, ws,
-                       reinterpret_cast<const uint4 *>(a.act8), a.mvals, a.u, a.M, a.Mp, n_units, nz,
+    hipLaunchKernelGGL((rq_skinny_kernel<TT, SINGLE, WIDE>), dim3(blocks), dim3(kThreads), 0, stream, ws,
+                       reinterpret_cast<const uint4 *>(a.act8), a.mvals, a.u, a.M, a.Mp, gsh, n_units, nz,
                        reinterpret_cast<unsigned long long *>(a.tot), ws.first[kMaxFused] * kPanelRows,
-                       plan.main_panels, plan.tail_split, ws.ng / plan.tail_split, ws.ng % plan.tail_split,
+                       plan.main_panels, plan.tail_split, n_groups / plan.tail_split, n_groups % plan.tail_split,
                        a.panels > 0 ? a.panel0 : 0);
     return hipGetLastError();
 }
@@ -343,10 +408,12 @@ hipError_t launch_tt(const SkinnyArgs &a, hipStream_t stream) {
 // whole rounds run as whole-K workgroups, and the remainder is cut along K into slices small enough to spread over
 // the chip: `tail_split` slices per panel, which meet in 64-bit arrival cells. Device-scope atomics cost about 7 ns
 // per thousand, so the cut is chosen by a small cost model (busiest compute unit + atomics) rather than maximised.
-SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz) {
+SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz, int runs_per_group) {
     const int kCUs = device_compute_units();
     SkinnyPlan plan;
-    const int smax = ng / 4 < 1 ? 1 : (ng / 4 > 16 ? 16 : ng / 4);   // at least four groups per slice
+    // at least four runs of 64 per slice, and whole activation groups (runs_per_group runs each)
+    const int per_slice = runs_per_group > 4 ? runs_per_group : 4;
+    const int smax = ng / per_slice < 1 ? 1 : (ng / per_slice > 16 ? 16 : ng / per_slice);
     const int per_round = kCUs / nz;                       // panels in one round of the chip
     plan.main_panels = n_panels / per_round * per_round;
     plan.tail_split = 1;
@@ -372,6 +439,11 @@ SkinnyPlan skinny_plan(int n_panels, int ng, int M, int nz) {
 hipError_t launch_skinny(const SkinnyArgs &a, hipStream_t stream) {
     constexpr int tt1_max = 16;   // most tokens served with one token tile of 16 per wavefront
     if (a.panels > 0) return launch_tt<2, false>(a, stream);   // the tail of a GEMM launch: blocks of 32 tokens
+    if (a.mvals != nullptr && a.runs_per_group > 1) {
+        // activation groups of 128 / 256: one or two token tiles per wavefront, more tokens as blocks of 32
+        if (a.M <= 16) return launch_tt<1, true, true>(a, stream);
+        return launch_tt<2, true, true>(a, stream);
+    }
     if (a.mvals != nullptr) {   // the caller wrote single-plane activations
         // 33..64 tokens: one workgroup with four token tiles per wavefront reads the weights once and halves the
         // workgroup count, two blocks of 32 tokens give twice the workgroups. The former wins on long rows and on
