@@ -202,6 +202,15 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         red[tid] = 0;
     }
     if (tid == 0) s_cnt[0] = 0;
+    // The first of the kernel's two hardware barriers (the other one stands in front of the epilogue): the cells and
+    // the phase counter are initialized before anybody adds to them. It comes early, where no wavefront is held up by the memory queue yet. The stream wavefronts do NOT wait
+    // for the row: a compute unit's memory pipeline takes requests in issue order, and the row was requested by the
+    // kernel's first instructions, so it is ahead of every weight by construction. (When the row was requested
+    // further down, weight requests that got in front of it delayed it by the translation of their first page:
+    // with 1, 2, 4 or 9 of a wavefront's 10 groups requested early the call took 11.9, 11.7, 12.5, 15.3 us instead of
+    // 11.0, and a barrier held the stream back until the row had arrived. With the row first, that barrier only
+    // cost time: 8.5 -> 7.7 us at N = 5120.)
+    __builtin_amdgcn_s_barrier();
 
     if (wave >= kRotWaves) {
         // =========================================================== the weight stream
@@ -213,11 +222,6 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         const int32_t f1 = __builtin_nontemporal_load(a.ws.flags[1]);
         const int32_t f2 = __builtin_nontemporal_load(a.ws.flags[2]);
 
-        // Behind this barrier the rotate wavefronts have the row. Not one weight is requested before: with 1, 2, 4
-        // or 9 of a wavefront's 10 groups ahead of the barrier the row arrives later and the whole call takes 11.9,
-        // 11.7, 12.5 and 15.3 us instead of 11.0; even a single 4-byte read per wavefront (to have the weight pages
-        // translated early) costs 0.5 us, because a wavefront's loads return in order and that first one is slow.
-        __builtin_amdgcn_s_barrier();
         RQ_STAMP(1);
 
         const bool anyk = ((f0 | f1 | f2) & 1) != 0;
@@ -393,10 +397,8 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         // =========================================================== the activation side (512 threads)
         const int rt = tid;
         int sync_target = 0;
-        // The stream starts only when the row has ARRIVED: requests queued behind the weight stream are served
-        // after it (a row requested just before the stream took 5 us instead of 1.5).
+        // the row (requested at the top of the kernel)
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
         RQ_STAMP(1);
 #pragma unroll
         for (int ub = 0; ub < kUnits; ++ub) {

@@ -19,7 +19,7 @@ from ruquant_amd import synth  # noqa: E402
 
 ROTATE = ["entry", "row arrived", "Sylvester done, row in LDS", "(LDS passes)", "Paley done", "group ranges",
           "codes in LDS", "stream finished"]
-STREAM = ["entry", "barrier: row arrived", "all loads issued", "codes seen", "last group folded", "cells complete"]
+STREAM = ["entry", "flag words requested", "all loads issued", "codes seen", "last group folded", "cells complete"]
 
 
 def main():
