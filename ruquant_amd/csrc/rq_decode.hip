@@ -159,6 +159,19 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
     float *s_unit = s_part + kRotWaves;
     int *s_cnt = reinterpret_cast<int *>(s_unit + 1);   // phases the rotate wavefronts have finished, x kRotWaves
 
+    if (tid < kDecodeCells + 8) red[tid] = 0;
+    if (tid == 0) s_cnt[0] = 0;
+    // The first of the kernel's two hardware barriers (the other one stands in front of the epilogue): the cells and
+    // the phase counter are initialized before anybody adds to them. It comes early (behind the row request, in front
+    // of everything that needs more arguments), where no wavefront is held up yet. The stream wavefronts do NOT wait
+    // for the row: a compute unit's memory pipeline takes requests in issue order, and the row was requested by the
+    // kernel's first instructions, so it is ahead of every weight by construction. (When the row was requested
+    // further down, weight requests that got in front of it delayed it by the translation of their first page:
+    // with 1, 2, 4 or 9 of a wavefront's 10 groups requested early the call took 11.9, 11.7, 12.5, 15.3 us instead of
+    // 11.0, and a barrier held the stream back until the row had arrived. With the row first, that barrier only
+    // cost time: 8.5 -> 7.7 us at N = 5120.)
+    __builtin_amdgcn_s_barrier();
+
     // ---- this workgroup's rows: whole panels s, s + G, ..., and a run of quads of the remainder panels. Remainder
     // slots run over the XCDs so that slots t and t + 1 (which may share an octet) sit on one XCD: workgroups go to
     // the eight XCDs round robin.
@@ -199,18 +212,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
             pre_sw = s_w[n];
             y_row = y + n;
         }
-        red[tid] = 0;
     }
-    if (tid == 0) s_cnt[0] = 0;
-    // The first of the kernel's two hardware barriers (the other one stands in front of the epilogue): the cells and
-    // the phase counter are initialized before anybody adds to them. It comes early, where no wavefront is held up by the memory queue yet. The stream wavefronts do NOT wait
-    // for the row: a compute unit's memory pipeline takes requests in issue order, and the row was requested by the
-    // kernel's first instructions, so it is ahead of every weight by construction. (When the row was requested
-    // further down, weight requests that got in front of it delayed it by the translation of their first page:
-    // with 1, 2, 4 or 9 of a wavefront's 10 groups requested early the call took 11.9, 11.7, 12.5, 15.3 us instead of
-    // 11.0, and a barrier held the stream back until the row had arrived. With the row first, that barrier only
-    // cost time: 8.5 -> 7.7 us at N = 5120.)
-    __builtin_amdgcn_s_barrier();
 
     if (wave >= kRotWaves) {
         // =========================================================== the weight stream
