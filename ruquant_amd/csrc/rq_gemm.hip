@@ -45,15 +45,25 @@ typedef __attribute__((address_space(1))) const void global_cvoid;
 
 constexpr int kBT = 128;        // tokens per workgroup, wide tiles
 constexpr int kBTn = 32;        // tokens per workgroup, narrow tiles
+constexpr int kBTh = 64;        // tokens per workgroup, half tiles
 constexpr int kThreads = 512;
 constexpr int kStages = 6;      // LDS ring depth
-constexpr int kLoads = 3;       // LDS-direct loads per thread and step (both tile shapes)
+
+// Tile shapes (the kernel's template argument). All are 256 rows; a wavefront owns 64 rows x TT token tiles of 16.
+//   kWide  : 128 tokens, wavefront columns = token halves of 64
+//   kNarrow:  32 tokens, wavefront columns = alternate groups of K (they meet in LDS at the end)
+//   kHalf  :  64 tokens, wavefront columns = token halves of 32: the wide tile's data flow at half its width, for
+//             launches whose wide tiles would not fill one round of the chip
+constexpr int kWide = 0, kNarrow = 1, kHalf = 2;
+constexpr int tiles_of(int mode) { return mode == kWide ? 4 : 2; }          // token tiles of 16 per wavefront
+constexpr int loads_of(int mode) { return mode == kHalf ? 2 : 3; }          // LDS-direct loads per thread and step
 
 // One ring stage = 1536 cells of 16 bytes = 24 KiB.
 //   wide tile  : [0, 512)    packed weights of one group  [panel 4][half 2][row 64]
 //                [512, 1536) activation digits            [digit 2][quarter 4][token 128]
 //   narrow tile: [0, 1024)   packed weights of two groups [group 2][panel 4][half 2][row 64]
 //                [1024,1536) activation digits            [group 2][digit 2][quarter 4][token 32]
+//   half tile  : [0, 512)    packed weights of one group; [512, 1024) activation digits [digit 2][quarter 4][token 64]
 struct Stage {
     uint4 cell[1536];
 };
@@ -90,10 +100,14 @@ __device__ __forceinline__ void load_to_lds(const uint4 *gptr, uint4 *lds) {
 
 // fetch of step `st` into stage s: every wavefront moves three 1 KiB runs. Groups past the end are clamped to the
 // last one (refetched into cells nobody reads).
-template <bool NARROW>
+template <int MODE>
 __device__ __forceinline__ void fetch(const Ctx &c, Stage &s, int st) {
     uint4 *dst = &s.cell[0] + c.wave * 64;
-    if (!NARROW) {
+    if (MODE == kHalf) {
+        const int g = st < c.ng ? st : c.ng - 1;
+        load_to_lds(c.w_src + (size_t) g * 128, dst);
+        load_to_lds(c.a_src + (size_t) g * c.a_step, dst + 512);   // both digits: thread tid moves cell tid of 512
+    } else if (MODE == kWide) {
         const int g = st < c.ng ? st : c.ng - 1;
         load_to_lds(c.w_src + (size_t) g * 128, dst);
         load_to_lds(c.a_src + (size_t) g * c.a_step, dst + 512);
@@ -110,18 +124,20 @@ __device__ __forceinline__ void fetch(const Ctx &c, Stage &s, int st) {
 
 // One step of one wavefront: 64 rows x TT token tiles of 16 against one group (wide: group `st`, token half wc;
 // narrow: group 2 st + wc).
-template <bool HASK, bool NARROW>
+template <bool HASK, int MODE>
 __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint8_t *__restrict__ k_src, int st,
-                                        v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
-    constexpr int TT = NARROW ? 2 : 4;
+                                        v4i (&hi)[4][tiles_of(MODE)], int32_t (&lo)[4][tiles_of(MODE)][4]) {
+    constexpr bool NARROW = MODE == kNarrow;
+    constexpr int TT = tiles_of(MODE);
     const int g = NARROW ? 2 * st + c.wc : st;
     if (NARROW && g >= c.ng) return;   // odd group count: the second K half sits out the last step (wave-uniform)
     // A: quarter `quad` of the group = 8 bytes of the row's cell in half quad >> 1
     const uint4 *a_cells = &s.cell[0] + (NARROW ? c.wc * 512 : 0) + (c.wr * 2 + (c.quad >> 1)) * 64 + c.l16;
     // B: [digit][quarter][token]
-    const uint4 *b_cells = NARROW ? &s.cell[1024] + c.wc * 256 + c.quad * kBTn + c.l16
-                                  : &s.cell[512] + c.quad * kBT + 64 * c.wc + c.l16;
-    constexpr int kDigit = NARROW ? 4 * kBTn : 4 * kBT;   // cells between the lo and the hi plane
+    const uint4 *b_cells = NARROW         ? &s.cell[1024] + c.wc * 256 + c.quad * kBTn + c.l16
+                           : MODE == kHalf ? &s.cell[512] + c.quad * kBTh + 32 * c.wc + c.l16
+                                           : &s.cell[512] + c.quad * kBT + 64 * c.wc + c.l16;
+    constexpr int kDigit = NARROW ? 4 * kBTn : MODE == kHalf ? 4 * kBTh : 4 * kBT;   // cells between the lo and the hi plane
     v4i A[4];
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
@@ -189,13 +205,16 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, const uint
 
 // Two groups of a tile at once (the fast path: no weight multipliers), in units of one 16 x 16 tile (x two groups =
 // 4 MFMAs); the second group of a unit is issued one unit later, when the first group's result has arrived.
-template <bool NARROW>
+template <int MODE>
 __device__ __forceinline__ void compute_pair(const Ctx &c, const Stage &sa, const Stage &sb,
-                                             v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
-    constexpr int TT = NARROW ? 2 : 4;
-    constexpr int kDigit = NARROW ? 4 * kBTn : 4 * kBT;   // cells between the lo and the hi plane
+                                             v4i (&hi)[4][tiles_of(MODE)], int32_t (&lo)[4][tiles_of(MODE)][4]) {
+    constexpr bool NARROW = MODE == kNarrow;
+    constexpr int TT = tiles_of(MODE);
+    constexpr int kDigit = NARROW ? 4 * kBTn : MODE == kHalf ? 4 * kBTh : 4 * kBT;   // cells between the lo and the hi plane
     const int a_off = (NARROW ? c.wc * 512 : 0) + (c.wr * 2 + (c.quad >> 1)) * 64 + c.l16;
-    const int b_off = NARROW ? 1024 + c.wc * 256 + c.quad * kBTn + c.l16 : 512 + c.quad * kBT + 64 * c.wc + c.l16;
+    const int b_off = NARROW         ? 1024 + c.wc * 256 + c.quad * kBTn + c.l16
+                      : MODE == kHalf ? 512 + c.quad * kBTh + 32 * c.wc + c.l16
+                                      : 512 + c.quad * kBT + 64 * c.wc + c.l16;
     v4i Aa[4], Ab[4];
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
@@ -309,16 +328,16 @@ __device__ __forceinline__ void compute_units(const Ctx &c, const Stage &cur0, c
 
 // One pair of steps: wait for their operands, meet the other wavefronts, refill the two stages that were just
 // released, compute. At the wait, the loads this thread has issued after this pair's are those of the next pair.
-template <bool HASK, bool NARROW>
+template <bool HASK, int MODE>
 __device__ __forceinline__ void pair_step(const Ctx &c, const Stage &cur0, const Stage &cur1, Stage &refill0,
                                           Stage &refill1, const uint8_t *__restrict__ k_src, int st, int n_steps,
-                                          v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoads) : "memory");
+                                          v4i (&hi)[4][tiles_of(MODE)], int32_t (&lo)[4][tiles_of(MODE)][4]) {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * loads_of(MODE)) : "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    fetch<NARROW>(c, refill0, st + 4);
-    fetch<NARROW>(c, refill1, st + 5);
-    if constexpr (NARROW) {
+    fetch<MODE>(c, refill0, st + 4);
+    fetch<MODE>(c, refill1, st + 5);
+    if constexpr (MODE == kNarrow) {
         if (c.gs > 1) {
             compute_units<HASK>(c, cur0, cur1, k_src, st, hi, lo);
             return;
@@ -327,26 +346,26 @@ __device__ __forceinline__ void pair_step(const Ctx &c, const Stage &cur0, const
     if constexpr (!HASK) {
         // K is a multiple of 256, so the number of groups is a multiple of 4: a pair of steps (two groups wide, four
         // narrow) is always whole
-        compute_pair<NARROW>(c, cur0, cur1, hi, lo);
+        compute_pair<MODE>(c, cur0, cur1, hi, lo);
     } else {
-        compute<HASK, NARROW>(c, cur0, k_src, st, hi, lo);
-        if (st + 1 < n_steps) compute<HASK, NARROW>(c, cur1, k_src, st + 1, hi, lo);
+        compute<HASK, MODE>(c, cur0, k_src, st, hi, lo);
+        if (st + 1 < n_steps) compute<HASK, MODE>(c, cur1, k_src, st + 1, hi, lo);
     }
 }
 
-template <bool HASK, bool NARROW>
+template <bool HASK, int MODE>
 __device__ __forceinline__ void gemm_body(const Ctx &c, Stage &s0, Stage &s1, Stage &s2, Stage &s3, Stage &s4,
                                           Stage &s5, const uint8_t *__restrict__ k_src,
-                                          v4i (&hi)[4][NARROW ? 2 : 4], int32_t (&lo)[4][NARROW ? 2 : 4][4]) {
-    const int n_steps = NARROW ? (c.ng + 1) / 2 : c.ng;
-    fetch<NARROW>(c, s0, 0);
-    fetch<NARROW>(c, s1, 1);
-    fetch<NARROW>(c, s2, 2);
-    fetch<NARROW>(c, s3, 3);
+                                          v4i (&hi)[4][tiles_of(MODE)], int32_t (&lo)[4][tiles_of(MODE)][4]) {
+    const int n_steps = MODE == kNarrow ? (c.ng + 1) / 2 : c.ng;
+    fetch<MODE>(c, s0, 0);
+    fetch<MODE>(c, s1, 1);
+    fetch<MODE>(c, s2, 2);
+    fetch<MODE>(c, s3, 3);
     for (int st = 0; st < n_steps; st += kStages) {
-        pair_step<HASK, NARROW>(c, s0, s1, s4, s5, k_src, st, n_steps, hi, lo);
-        if (st + 2 < n_steps) pair_step<HASK, NARROW>(c, s2, s3, s0, s1, k_src, st + 2, n_steps, hi, lo);
-        if (st + 4 < n_steps) pair_step<HASK, NARROW>(c, s4, s5, s2, s3, k_src, st + 4, n_steps, hi, lo);
+        pair_step<HASK, MODE>(c, s0, s1, s4, s5, k_src, st, n_steps, hi, lo);
+        if (st + 2 < n_steps) pair_step<HASK, MODE>(c, s2, s3, s0, s1, k_src, st + 2, n_steps, hi, lo);
+        if (st + 4 < n_steps) pair_step<HASK, MODE>(c, s4, s5, s2, s3, k_src, st + 4, n_steps, hi, lo);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the refetches of the last steps before LDS is reused
 }
@@ -355,7 +374,7 @@ __device__ __forceinline__ void gemm_body(const Ctx &c, Stage &s0, Stage &s1, St
 // ceil(T / 256) rounds. So only whole rounds (or none, or all: see launch_gemm) run wide, and the rest (`first_tile`
 // onwards) run as narrow tiles: the same 256 rows x 32 tokens, with the two wavefront columns taking alternate groups of K instead of
 // token halves and meeting in LDS at the end. Four times as many workgroups of a quarter of the work each.
-template <bool NARROW>
+template <int MODE>
 __global__ void __launch_bounds__(kThreads)
 rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                const int32_t *__restrict__ flags, const uint4 *__restrict__ act8, const float *__restrict__ u,
@@ -368,7 +387,9 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     __shared__ Stage s3;
     __shared__ Stage s4;
     __shared__ Stage s5;
-    constexpr int TT = NARROW ? 2 : 4;
+    constexpr bool NARROW = MODE == kNarrow;
+    constexpr int TT = tiles_of(MODE);
+    constexpr int kTok = MODE == kHalf ? kBTh : kBT;   // tokens of a wide or half tile
 
     // Workgroups go to the eight XCDs round robin. Wide: give every XCD a contiguous run of row tiles with the token
     // tiles running fastest, so the workgroups resident on one XCD share weight and activation tiles in its L2.
@@ -385,10 +406,10 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
             const int spr = n_tok_tiles >> 2;
             const int sr = s / spr;
             row_tile = sr * 8 + (i >> 2);
-            t0 = ((s - sr * spr) * 4 + (i & 3)) * kBT;
+            t0 = ((s - sr * spr) * 4 + (i & 3)) * kTok;
         } else {
             row_tile = v / n_tok_tiles;
-            t0 = (v - row_tile * n_tok_tiles) * kBT;
+            t0 = (v - row_tile * n_tok_tiles) * kTok;   // (half tiles: n_tok_tiles counts tiles of 64 tokens)
         }
     } else {
         // Narrow workgroups cover whole row tiles from `first_tile / n_tok_tiles` on; only token quarters that hold
@@ -418,7 +439,11 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     c.w_src = codes + (size_t) w_panel * ng * 128 + (tid & 127);
     c.a_step = (size_t) 8 * Mp;   // cells per group
     c.a_cell = (size_t) 4 * Mp;   // the other digit
-    if (!NARROW) {
+    if (MODE == kHalf) {
+        // the tile of one group is 512 cells [digit][quarter][token 64]; thread tid moves cell tid (digit and quarter =
+        // tid >> 6, which is also their order in the planes)
+        c.a_src = act8 + (size_t) (tid >> 6) * Mp + t0 + (tid & 63);
+    } else if (!NARROW) {
         // the tile of one group is 1024 cells [digit][quarter][token]; thread tid moves cells tid and tid + 512
         // (digit = cell >> 9, quarter = (cell >> 7) & 3, token = cell & 127)
         c.a_src = act8 + (size_t) (tid >> 7) * Mp + t0 + (tid & 127);
@@ -442,9 +467,9 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     }
 
     if (flags[0] & 1) {
-        gemm_body<true, NARROW>(c, s0, s1, s2, s3, s4, s5, k_src, hi, lo);
+        gemm_body<true, MODE>(c, s0, s1, s2, s3, s4, s5, k_src, hi, lo);
     } else {
-        gemm_body<false, NARROW>(c, s0, s1, s2, s3, s4, s5, k_src, hi, lo);
+        gemm_body<false, MODE>(c, s0, s1, s2, s3, s4, s5, k_src, hi, lo);
     }
 
     // (the fast path leaves the sum of the floors in the bits above the low byte: see compute_pair)
@@ -489,7 +514,7 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     // epilogue (reference patch line 176): y = ((float(total) * 16) * u) * s_w, total = 4 Xhi + sum of floors
 #pragma unroll
     for (int ct = 0; ct < TT; ++ct) {
-        const int t = t0 + (NARROW ? 0 : 64 * c.wc) + 16 * ct + c.l16;
+        const int t = t0 + (NARROW ? 0 : MODE == kHalf ? 32 * c.wc : 64 * c.wc) + 16 * ct + c.l16;
         if (t >= M) continue;
         const float ut = u[t];
 #pragma unroll
@@ -519,6 +544,8 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
 
 }  // namespace
 
+constexpr double kHalfRound = 1.5;   // a round of half tiles, in rounds of narrow tiles
+
 hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     const uint8_t *p = a.prepared;
     const int n_row_tiles = (a.L.n_panels + 3) / 4;
@@ -545,17 +572,25 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     // each: it wins when the leftover is a few row tiles and the token count moderate (K=5120, N=17408, M=512: 256
     // wide tiles + 16 panels x 16 token blocks, 116.6 -> 102.4 us; at M=1024 the narrow tiles stay ahead).
     bool skinny_tail = false;
+    double best = cost(n_wide);
     // (the skinny kernel addresses the digit planes with 32-bit offsets)
     const bool planes_fit = (int64_t) a.L.ng * 128 * a.Mp < ((int64_t) 1 << 32);
     if (a.groups_per_fold == 1 && whole > 0 && whole < n_tiles && planes_fit) {
         const int tail_panels = a.L.n_panels - whole / n_tok_tiles * 4;
         const int64_t wgs = (int64_t) tail_panels * ((a.M + 31) / 32);
         const double c = 2.6 * (whole / kCUs) + 0.65 * ((wgs + kCUs - 1) / kCUs);
-        if (c < cost(n_wide)) {
+        if (c < best) {
             n_wide = whole;
             skinny_tail = true;
+            best = c;
         }
     }
+    // A fourth way: half tiles (256 rows x 64 tokens) for the whole launch, when that many tiles fill the rounds of
+    // the chip better than the mixes above (K = 5120, N = 6144, M = 512: 192 half tiles in one round against 384
+    // narrow tiles in two). A round of half tiles takes about 1.5 rounds of narrow ones (46 us against 31 us at K = 5120).
+    const int n_half_tok = (a.M + kBTh - 1) / kBTh;
+    const int n_half = n_row_tiles * n_half_tok;
+    const bool half_tiles = a.groups_per_fold == 1 && kHalfRound * ((n_half + kCUs - 1) / kCUs) < best;
     // the super-tile order of the wide kernel needs a wide region of whole blocks of 8 row tiles x 4 token tiles
     const int super_tiles = n_wide > 0 && n_tok_tiles % 4 == 0 && n_wide % n_tok_tiles == 0 &&
                             (n_wide / n_tok_tiles) % 8 == 0;
@@ -563,8 +598,14 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     const float *s_w = reinterpret_cast<const float *>(p + a.L.off_sw);
     const int32_t *flags = reinterpret_cast<const int32_t *>(p + a.L.off_flags);
     const uint4 *act8 = reinterpret_cast<const uint4 *>(a.act8);
+    if (half_tiles) {
+        hipLaunchKernelGGL(rq_gemm_kernel<kHalf>, dim3(n_half), dim3(kThreads), 0, stream, codes, s_w,
+                           p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
+                           n_half_tok, 0, n_half, 0, 4);
+        return hipGetLastError();
+    }
     if (n_wide > 0) {
-        hipLaunchKernelGGL(rq_gemm_kernel<false>, dim3(n_wide), dim3(kThreads), 0, stream, codes, s_w,
+        hipLaunchKernelGGL(rq_gemm_kernel<kWide>, dim3(n_wide), dim3(kThreads), 0, stream, codes, s_w,
                            p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
                            n_tok_tiles, 0, n_wide, super_tiles, 4);
     }
@@ -587,7 +628,7 @@ hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream) {
     }
     if (n_wide < n_tiles) {
         const int n_blocks = (n_row_tiles - n_wide / n_tok_tiles) * per_row;
-        hipLaunchKernelGGL(rq_gemm_kernel<true>, dim3(n_blocks), dim3(kThreads), 0, stream, codes, s_w,
+        hipLaunchKernelGGL(rq_gemm_kernel<kNarrow>, dim3(n_blocks), dim3(kThreads), 0, stream, codes, s_w,
                            p + a.L.off_kmul, flags, act8, a.u, a.y, a.ldy, a.L.N, a.M, a.Mp, a.L.ng, a.L.n_panels,
                            n_tok_tiles, n_wide, n_blocks, a.groups_per_fold, live_last);
     }

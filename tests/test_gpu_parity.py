@@ -167,6 +167,20 @@ def test_mul_mat_longest_row(oracle, type_, M):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
+@pytest.mark.parametrize("N,K,M,wgroup,type_", [(6144, 1024, 512, 0, rq.TYPE_W4A4H), (6100, 1536, 500, 0, rq.TYPE_W4A4H),
+                                                (6144, 1024, 450, 256, rq.TYPE_W4A4), (6144, 768, 512, 64, rq.TYPE_W4A4H)])
+def test_gemm_half_tiles(oracle, N, K, M, wgroup, type_):
+    """Shapes whose wide tiles would not fill one round of the chip and whose narrow tiles need two: the launch plan
+    runs them as half tiles (256 rows x 64 tokens; 24 row tiles x 8 token tiles = 192 workgroups). Whole and ragged
+    token and row counts, with and without weight multipliers."""
+    blocks, wf = adversarial_weights(oracle, N, K, type_, wgroup=wgroup)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    x = adversarial_activations(M, K, type_, wf, seed=M)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=max(W.n_rot, 0))
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
 def test_gemm_wide_tiles_longest_row_extreme_sums(oracle):
     """K = 32768 on the wide tiles of the MFMA GEMM with inputs that drive the integer sums to their ends: rows whose
     codes are all -8 or all +7 against tokens that quantize to q - z = +15 or -15 with m = 255 in every one of the
