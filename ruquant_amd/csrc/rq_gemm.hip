@@ -22,7 +22,8 @@
 // accumulators every group and fold floor(k (64 Xhi + Xlo) / 16) on the vector ALU.
 //
 // Data movement: a workgroup of eight wavefronts owns 256 rows (four panels) x 128 tokens; wavefront (wr, wc) owns
-// rows 64 wr.. and tokens 64 wc.. as 4 x 4 MFMA tiles (a narrow variant for the tail of a launch: see the kernel). The operands of one group (8 KiB of packed weights, 16 KiB of
+// rows 64 wr.. and tokens 64 wc.. as 4 x 4 MFMA tiles (narrow and half-width variants for launches and tails that wide
+// tiles do not fill: see the tile shapes below and launch_gemm). The operands of one group (8 KiB of packed weights, 16 KiB of
 // activation digits) go from global memory straight into LDS with global_load_lds_dwordx4 (no registers, no
 // ds_write), kStages groups deep, so a fetch has several groups of arithmetic to complete. The prepared weight
 // layout and the quantizer's output layout are exactly the LDS layouts: every wavefront-wide transfer is 1 KiB
