@@ -14,8 +14,10 @@ class LibraryMissing(RuntimeError):
 
 
 def build_library(jobs=8):
-    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU)."""
-    subprocess.run(["make", "-C", CSRC, "-B", "-j%d" % jobs], check=True)
+    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU): the library, the host program and the
+    instrumented build of the decode kernel that ruquant_amd/decode_stamps.py loads."""
+    subprocess.run(["make", "-C", CSRC, "-B", "-j%d" % jobs, "all"], check=True)
+    subprocess.run(["make", "-C", CSRC, "stamps"], check=True)
     return LIB_PATH
 
 
