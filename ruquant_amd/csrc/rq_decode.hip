@@ -31,6 +31,8 @@
 __device__ unsigned long long rq_decode_stamps[64];
 #define RQ_STAMP_DECL unsigned long long rq_st[8] = {}
 #define RQ_STAMP(i) do { rq_st[(i)] = __builtin_readcyclecounter(); } while (0)
+#define RQ_STAMP_AT(st, i) do { (st)[(i)] = __builtin_readcyclecounter(); } while (0)
+#define RQ_STAMP_PTR rq_st
 #define RQ_STAMP_FLUSH do { if (blockIdx.x == 0 && (threadIdx.x == 0 || threadIdx.x == 512)) { \
         for (int i_ = 0; i_ < 8; ++i_) rq_decode_stamps[i_ + (threadIdx.x ? 32 : 0)] = rq_st[i_]; } } while (0)
 extern "C" int rq_w4a4_decode_stamps(unsigned long long *out) {
@@ -39,6 +41,8 @@ extern "C" int rq_w4a4_decode_stamps(unsigned long long *out) {
 #else
 #define RQ_STAMP_DECL do { } while (0)
 #define RQ_STAMP(i) do { } while (0)
+#define RQ_STAMP_AT(st, i) do { } while (0)
+#define RQ_STAMP_PTR nullptr
 #define RQ_STAMP_FLUSH do { } while (0)
 #endif
 
@@ -105,6 +109,83 @@ __device__ __forceinline__ void rot_sync(int *cnt, int &target, int lane) {
     if (lane == 0) atomicAdd(cnt, 1);
     target += kRotWaves;
     wait_count<false>(cnt, target);
+}
+
+// The activation quantizer of the rotate wavefronts for R code words per thread (word w = r x 512 + thread, its eight
+// values stay in registers between the two phases): group ranges [min(x, 0), max(x, 0)] x clip with eight lanes per
+// group of 64 and the token's widest range (reference lines 2646-2654); then, behind the phase barrier, the unit, per
+// group multiplier and zero point, and the 4-bit codes (reference lines 2662-2677). R is a compile-time constant so
+// that the R rounds are one instruction stream: their LDS reads go out together and their dependent min / max / DPP
+// chains interleave (as separate uniform branches the rounds ran one after the other).
+template <int R>
+__device__ __forceinline__ void quantize_rounds(const float *row, bool dense, int nw, float clip, int rt, int lane,
+                                                int wave, float *s_part, float *s_unit, uint32_t *s_act,
+                                                int32_t *s_mz, int *s_cnt, int &sync_target, unsigned long long *stamps) {
+    (void) stamps;
+    float f[R][8];
+    float g_lo_r[R], g_hi_r[R];
+#pragma unroll
+    for (int wr = 0; wr < R; ++wr) {
+        const int w = wr * kRotThreads + rt;
+        const bool on = w < nw;
+        if (dense) {
+            const float4 *sp = reinterpret_cast<const float4 *>(row + 8 * (on ? w : 0));
+            const float4 v0 = sp[0], v1 = sp[1];
+            f[wr][0] = v0.x; f[wr][1] = v0.y; f[wr][2] = v0.z; f[wr][3] = v0.w;
+            f[wr][4] = v1.x; f[wr][5] = v1.y; f[wr][6] = v1.z; f[wr][7] = v1.w;
+        } else {
+            const float *sp = row + padi(8 * (on ? w : 0));
+#pragma unroll
+            for (int j = 0; j < 8; ++j) f[wr][j] = sp[j];
+        }
+        if (!on) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) f[wr][j] = 0.0f;
+        }
+    }
+    float rmax = 0.0f;
+#pragma unroll
+    for (int wr = 0; wr < R; ++wr) {
+        const bool on = wr * kRotThreads + rt < nw;
+        float mn = fminf(fminf(fminf(fminf(0.0f, f[wr][0]), fminf(f[wr][1], f[wr][2])),
+                               fminf(fminf(f[wr][3], f[wr][4]), fminf(f[wr][5], f[wr][6]))), f[wr][7]);
+        float mx = fmaxf(fmaxf(fmaxf(fmaxf(0.0f, f[wr][0]), fmaxf(f[wr][1], f[wr][2])),
+                               fmaxf(fmaxf(f[wr][3], f[wr][4]), fmaxf(f[wr][5], f[wr][6]))), f[wr][7]);
+        mn = group8_reduce<false>(mn);
+        mx = group8_reduce<true>(mx);
+        g_lo_r[wr] = mn * clip;
+        g_hi_r[wr] = mx * clip;
+        if (on) rmax = fmaxf(rmax, g_hi_r[wr] - g_lo_r[wr]);
+    }
+    rmax = wave_max(rmax);
+    if (lane == 0) s_part[wave] = rmax;
+    rot_sync(s_cnt, sync_target, lane);
+    RQ_STAMP_AT(stamps, 5);
+
+    float Rg = s_part[0];
+#pragma unroll
+    for (int i = 1; i < kRotWaves; ++i) Rg = fmaxf(Rg, s_part[i]);
+    if (Rg == 0.0f) Rg = 2.0f;
+    const float u = Rg / 3825.0f;  // 15 * 255
+    if (rt == 0) s_unit[0] = u;
+#pragma unroll
+    for (int wr = 0; wr < R; ++wr) {
+        const int w = wr * kRotThreads + rt;
+        const float lo = g_lo_r[wr], hi = g_hi_r[wr];
+        const int mg = (int) fminf(fmaxf(ceilf(((hi - lo) * 255.0f) / Rg), 1.0f), 255.0f);
+        const float inv = 1.0f / ((float) mg * u);
+        const float zf = fminf(fmaxf(rintf(-lo * inv), 0.0f), 15.0f);
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int q = (int) fminf(fmaxf(rintf(f[wr][j] * inv) + zf, 0.0f), 15.0f);
+            word |= (uint32_t) ((q - 8) & 0xF) << (4 * j);
+        }
+        if (w < nw) {
+            s_act[w] = word;
+            if ((w & 7) == 0) s_mz[w >> 3] = mg | ((8 - (int) zf) & 0xFF) << 8;
+        }
+    }
 }
 
 // LDS: [row, padded][Paley output, dense][codes][mz][cells][wave maxima, unit, phase counter]
@@ -463,6 +544,29 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                 const int col_runs = (ncols + 63) >> 6;
                 const int n_it = kSlices * col_runs;
                 const int per_wave = (n_it + kRotWaves - 1) / kRotWaves;
+                if (per_wave == 2 && (col_runs & 1) == 0 && (ncols & 63) == 0 && 2 * wave + 1 < n_it) {
+                    // the wavefront's two items are neighbouring column runs of one slice: one instruction stream
+                    // for both (whole row rotated as H20 x H256 or H12 x H512: 16 items for eight wavefronts)
+                    int s = 0, cr = 2 * wave;
+                    while (cr >= col_runs) {
+                        cr -= col_runs;
+                        ++s;
+                    }
+                    const int c0 = cr * 64 + lane, c1 = c0 + 64;
+                    const int b0 = (c0 >> lm) * a.n_rot + (c0 & (m - 1)), b1 = (c1 >> lm) * a.n_rot + (c1 & (m - 1));
+                    float out0[kOut], out1[kOut];
+                    if (m == 256) {
+                        paley_pick_stream2<P, kOut, 272>(s, buf + padi(b0), buf + padi(b1), 272, out0, out1);
+                    } else {
+                        paley_pick_stream2<P, kOut, 0>(s, buf + padi(b0), buf + padi(b1), pm, out0, out1);
+                    }
+                    float *d0 = alt + b0 + kOut * s * m, *d1 = alt + b1 + kOut * s * m;
+#pragma unroll
+                    for (int o = 0; o < kOut; ++o) {
+                        d0[o * m] = out0[o] * a.scale;
+                        d1[o * m] = out1[o] * a.scale;
+                    }
+                } else
                 for (int it = 0; it < per_wave; ++it) {
                     const int wi = wave * per_wave + it;
                     if (wi >= n_it) break;
@@ -496,73 +600,17 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         }
 
         RQ_STAMP(4);
-        // ---- group ranges [min(x, 0), max(x, 0)] * clip and the token's widest range (reference lines 2646-2654):
-        // a thread per code word, eight lanes per group of 64; the word's eight values stay in registers for the codes
-        const int nw = K >> 3;
-        constexpr int kWordRounds = 4;   // K <= 16384
-        const bool dense = a.rotate && P > 1;            // the Paley stage wrote the dense buffer
-        float f[kWordRounds][8];
-        float g_lo_r[kWordRounds], g_hi_r[kWordRounds];
-        float rmax = 0.0f;
-#pragma unroll
-        for (int wr = 0; wr < kWordRounds; ++wr) {
-            const int w = wr * kRotThreads + rt;
-            if (wr * kRotThreads < nw) {   // uniform
-                const bool on = w < nw;
-                if (dense) {
-                    const float4 *sp = reinterpret_cast<const float4 *>(alt + 8 * (on ? w : 0));
-                    const float4 v0 = sp[0], v1 = sp[1];
-                    f[wr][0] = v0.x; f[wr][1] = v0.y; f[wr][2] = v0.z; f[wr][3] = v0.w;
-                    f[wr][4] = v1.x; f[wr][5] = v1.y; f[wr][6] = v1.z; f[wr][7] = v1.w;
-                } else {
-                    const float *sp = buf + padi(8 * (on ? w : 0));
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) f[wr][j] = sp[j];
-                }
-                if (!on) {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) f[wr][j] = 0.0f;
-                }
-                float mn = fminf(fminf(fminf(fminf(0.0f, f[wr][0]), fminf(f[wr][1], f[wr][2])),
-                                       fminf(fminf(f[wr][3], f[wr][4]), fminf(f[wr][5], f[wr][6]))), f[wr][7]);
-                float mx = fmaxf(fmaxf(fmaxf(fmaxf(0.0f, f[wr][0]), fmaxf(f[wr][1], f[wr][2])),
-                                       fmaxf(fmaxf(f[wr][3], f[wr][4]), fmaxf(f[wr][5], f[wr][6]))), f[wr][7]);
-                mn = group8_reduce<false>(mn);
-                mx = group8_reduce<true>(mx);
-                g_lo_r[wr] = mn * a.clip;
-                g_hi_r[wr] = mx * a.clip;
-                if (on) rmax = fmaxf(rmax, g_hi_r[wr] - g_lo_r[wr]);
-            }
-        }
-        rmax = wave_max(rmax);
-        if (lane == 0) s_part[wave] = rmax;
-        rot_sync(s_cnt, sync_target, lane);
-        RQ_STAMP(5);
-
-        float R = s_part[0];
-#pragma unroll
-        for (int i = 1; i < kRotWaves; ++i) R = fmaxf(R, s_part[i]);
-        if (R == 0.0f) R = 2.0f;
-        const float u = R / 3825.0f;  // 15 * 255
-        if (rt == 0) s_unit[0] = u;
-
-        // ---- per group multiplier and zero point, per value code (reference lines 2662-2677)
-#pragma unroll
-        for (int wr = 0; wr < kWordRounds; ++wr) {
-            const int w = wr * kRotThreads + rt;
-            if (wr * kRotThreads < nw && w < nw) {
-                const float lo = g_lo_r[wr], hi = g_hi_r[wr];
-                const int mg = (int) fminf(fmaxf(ceilf(((hi - lo) * 255.0f) / R), 1.0f), 255.0f);
-                const float inv = 1.0f / ((float) mg * u);
-                const float zf = fminf(fmaxf(rintf(-lo * inv), 0.0f), 15.0f);
-                uint32_t word = 0;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int q = (int) fminf(fmaxf(rintf(f[wr][j] * inv) + zf, 0.0f), 15.0f);
-                    word |= (uint32_t) ((q - 8) & 0xF) << (4 * j);
-                }
-                s_act[w] = word;
-                if ((w & 7) == 0) s_mz[w >> 3] = mg | ((8 - (int) zf) & 0xFF) << 8;
+        // ---- group ranges, the token's unit, multipliers, zero points and codes (quantize_rounds), with the number
+        // of code words per thread as a compile-time constant
+        {
+            const int nw = K >> 3;
+            const bool dense = a.rotate && P > 1;            // the Paley stage wrote the dense buffer
+            const float *row = dense ? alt : buf;
+            switch ((nw + kRotThreads - 1) / kRotThreads) {   // K <= 16384: at most four words per thread
+            case 1: quantize_rounds<1>(row, dense, nw, a.clip, rt, lane, wave, s_part, s_unit, s_act, s_mz, s_cnt, sync_target, RQ_STAMP_PTR); break;
+            case 2: quantize_rounds<2>(row, dense, nw, a.clip, rt, lane, wave, s_part, s_unit, s_act, s_mz, s_cnt, sync_target, RQ_STAMP_PTR); break;
+            case 3: quantize_rounds<3>(row, dense, nw, a.clip, rt, lane, wave, s_part, s_unit, s_act, s_mz, s_cnt, sync_target, RQ_STAMP_PTR); break;
+            default: quantize_rounds<4>(row, dense, nw, a.clip, rt, lane, wave, s_part, s_unit, s_act, s_mz, s_cnt, sync_target, RQ_STAMP_PTR); break;
             }
         }
         rot_sync(s_cnt, sync_target, lane);   // codes, multipliers and unit are in LDS: the stream folds

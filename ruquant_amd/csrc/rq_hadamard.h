@@ -92,6 +92,34 @@ __device__ __forceinline__ void paley_pick_stream(int s, const float *src, int s
     }
 }
 
+// The same for two columns at once (two runs of 64 columns of one slice): twice the independent sums per
+// instruction stream, which is what hides the latency of the dependent additions and of the LDS reads when a
+// wavefront has only two items.
+template <int P, int O, int STRIDE, int S = 0>
+__device__ __forceinline__ void paley_pick_stream2(int s, const float *src0, const float *src1, int stride,
+                                                   float (&out0)[O], float (&out1)[O]) {
+    if (s == S) {
+        constexpr PaleyTable<P> T = make_paley<P>();
+#pragma unroll
+        for (int o = 0; o < O; ++o) {
+            out0[o] = 0.0f;
+            out1[o] = 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < P; ++i) {
+            const float c0 = src0[i * (STRIDE ? STRIDE : stride)];
+            const float c1 = src1[i * (STRIDE ? STRIDE : stride)];
+#pragma unroll
+            for (int o = 0; o < O; ++o) {
+                out0[o] = T.neg[i][O * S + o] ? out0[o] - c0 : out0[o] + c0;
+                out1[o] = T.neg[i][O * S + o] ? out1[o] - c1 : out1[o] + c1;
+            }
+        }
+    } else if constexpr (S + 1 < P / O) {
+        paley_pick_stream2<P, O, STRIDE, S + 1>(s, src0, src1, stride, out0, out1);
+    }
+}
+
 // all P outputs of one column, written back in place (the column is private to the calling thread). STRIDE is the
 // distance between the chunks of a column in the padded row when it is known at compile time (0: use `stride`): the
 // P loads and P stores then share one or two address registers with immediate offsets, where a run-time stride costs
