@@ -212,7 +212,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
     // strides 16 .. 128 run between lanes and the row makes no trip through LDS between its stages. Lane l of a row
     // holds the unit whose index bits (b0, b1, b2, b3) give l = b0 ^ 2 b1 ^ 7 b2 ^ 8 b3: the partners of the four
     // stages are then l ^ 1, l ^ 2, l ^ 7, l ^ 8, which are single DPP controls.
-    const bool dpp256 = a.rotate && a.m == 256;
+    const bool dpp256 = a.rotate && (a.m & 255) == 0;   // chunks of whole blocks of 256 floats
     const int lr = lane & 15;
     const int hb3 = lr >> 3, hr = lr & 7, hb2 = hr >> 2, hr2 = hr ^ (hb2 ? 7 : 0);
     const int unit_of_lane = (hr2 & 1) | (hr2 & 2) | hb2 << 2 | hb3 << 3;
@@ -522,8 +522,10 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         if (a.rotate) {
             const int m = a.m;
             const int lm = __ffs(m) - 1;
-            if (!dpp256) {
-                for (int ls = 4; ls < lm;) {
+            {
+                // the stages behind the ones done in registers (strides 1 .. 8) and between lanes (16 .. 128, for
+                // chunks made of blocks of 256 floats), in ascending stride order through LDS
+                for (int ls = dpp256 ? 8 : 4; ls < lm;) {
                     const int lr2 = lm - ls < 4 ? lm - ls : 4;
                     if (lr2 == 4) fwht_pass<4>(buf, K, lm, ls, rt, kRotThreads);
                     else if (lr2 == 3) fwht_pass<3>(buf, K, lm, ls, rt, kRotThreads);
@@ -709,7 +711,10 @@ hipError_t launch_decode(const DecodeArgs &d, hipStream_t stream) {
     k.clip = d.clip;
     k.inv_nblk = (1 << 22) / (d.K / 256) + 1;
     const int lm = d.rotate ? __builtin_ctz((unsigned) d.m) : 0;
-    k.n_pass = d.rotate && lm > 4 && d.m != 256 ? (lm - 4 + 3) / 4 : 0;   // chunks of 256: the stages run between lanes
+    // stages through LDS: those above stride 8, or above stride 128 when the chunks are whole blocks of 256 floats
+    // (four more stages then run between lanes)
+    const int lm0 = d.rotate && (d.m & 255) == 0 ? 8 : 4;
+    k.n_pass = d.rotate && lm > lm0 ? (lm - lm0 + 3) / 4 : 0;
     const int n_panels = k.ws.first[kMaxFused];
     // one workgroup per compute unit: whole panels as far as they go round, the remainder in quads of rows. More
     // workgroups (a multiple of the compute units) only when the rows of one would not fit its LDS cells.
