@@ -82,20 +82,6 @@ __device__ __forceinline__ int align4(int v) { return (v + 3) & ~3; }
 // (The counter is read through an LDS-typed pointer: a generic one makes the poll a FLAT load, which queues behind
 // the weight stream.)
 typedef __attribute__((address_space(3))) int lds_int;
-// One Sylvester stage between lanes: `ctrl` swaps every lane with its partner (the lane whose unit differs in the
-// stage's index bit); the lane of the lower unit gets a + b, the upper one a - b with a the lower unit's value
-// (reference lines 2454-2464). t - v is formed as t + (-v): the same IEEE operation.
-template <int CTRL>
-__device__ __forceinline__ void dpp_stage(float (&v)[16], uint32_t upper_sign) {
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-        const float t = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v[j]), CTRL,
-                                                                              0xF, 0xF, false));
-        const float sv = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v[j]) ^ upper_sign);
-        v[j] = t + sv;
-    }
-}
-
 template <bool SLEEP>
 __device__ __forceinline__ void wait_count(const int *cnt, int target) {
     const volatile lds_int *c = (const volatile lds_int *) cnt;
@@ -209,13 +195,11 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
     // ---- the rotate wavefronts request the row before anything else: 16 consecutive floats per thread and unit.
     // Everything below (cells, row scales, item addresses) is computed while it travels.
     // Chunks of 256 floats (16 units): the 16 lanes of a DPP row hold one chunk, so the Sylvester stages with
-    // strides 16 .. 128 run between lanes and the row makes no trip through LDS between its stages. Lane l of a row
-    // holds the unit whose index bits (b0, b1, b2, b3) give l = b0 ^ 2 b1 ^ 7 b2 ^ 8 b3: the partners of the four
-    // stages are then l ^ 1, l ^ 2, l ^ 7, l ^ 8, which are single DPP controls.
+    // strides 16 .. 128 run between lanes and the row makes no trip through LDS between its stages (dpp_unit_of_lane
+    // says which unit a lane holds).
     const bool dpp256 = a.rotate && (a.m & 255) == 0;   // chunks of whole blocks of 256 floats
-    const int lr = lane & 15;
-    const int hb3 = lr >> 3, hr = lr & 7, hb2 = hr >> 2, hr2 = hr ^ (hb2 ? 7 : 0);
-    const int unit_of_lane = (hr2 & 1) | (hr2 & 2) | hb2 << 2 | hb3 << 3;
+    const DppUnit du = dpp_unit_of_lane(lane);
+    const int unit_of_lane = du.unit;
     constexpr int kUnits = 2;   // K <= 16384
     float4 qv[kUnits][4];
     if (wave < kRotWaves) {
@@ -505,12 +489,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                         }
                     }
                 }
-                if (dpp256) {
-                    dpp_stage<0xB1>(v, (uint32_t) (hr2 & 1) << 31);          // stride 16: quad_perm [1, 0, 3, 2]
-                    dpp_stage<0x4E>(v, (uint32_t) ((hr2 >> 1) & 1) << 31);   // stride 32: quad_perm [2, 3, 0, 1]
-                    dpp_stage<0x141>(v, (uint32_t) hb2 << 31);               // stride 64: row_half_mirror
-                    dpp_stage<0x128>(v, (uint32_t) hb3 << 31);               // stride 128: row_ror:8
-                }
+                if (dpp256) dpp_stages_256(v, du);   // strides 16 .. 128 between lanes
                 float *d = buf + padi(16 * u);
 #pragma unroll
                 for (int j = 0; j < 16; ++j) d[j] = v[j];

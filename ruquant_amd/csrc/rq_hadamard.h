@@ -342,6 +342,88 @@ __device__ __forceinline__ void load_row_fwht16(float *buf, const float *__restr
     }
 }
 
+// One Sylvester stage between lanes: `ctrl` swaps every lane with its partner (the lane whose unit differs in the
+// stage's index bit); the lane of the lower unit gets a + b, the upper one a - b with a the lower unit's value
+// (reference lines 2454-2464). t - v is formed as t + (-v): the same IEEE operation.
+template <int CTRL>
+__device__ __forceinline__ void dpp_stage(float (&v)[16], uint32_t upper_sign) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const float t = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v[j]), CTRL,
+                                                                              0xF, 0xF, false));
+        const float sv = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v[j]) ^ upper_sign);
+        v[j] = t + sv;
+    }
+}
+
+// The unit of 16 floats that lane `lane` of a DPP row of 16 lanes takes when the row holds one block of 256 floats: the
+// unit whose index bits (b0, b1, b2, b3) give lane = b0 ^ 2 b1 ^ 7 b2 ^ 8 b3, so that the partners of the stages with
+// strides 16, 32, 64, 128 are lane ^ 1, ^ 2, ^ 7, ^ 8: quad_perm, quad_perm, row_half_mirror and row_ror:8.
+struct DppUnit {
+    int unit;                 // 0 .. 15: the unit within the block of 256 floats
+    uint32_t s16, s32, s64, s128;   // sign bit of the lane's own value in each stage (set: upper partner, takes a - b)
+};
+__device__ __forceinline__ DppUnit dpp_unit_of_lane(int lane) {
+    const int lr = lane & 15;
+    const int hb3 = lr >> 3, hr = lr & 7, hb2 = hr >> 2, hr2 = hr ^ (hb2 ? 7 : 0);
+    DppUnit d;
+    d.unit = (hr2 & 1) | (hr2 & 2) | hb2 << 2 | hb3 << 3;
+    d.s16 = (uint32_t) (hr2 & 1) << 31;
+    d.s32 = (uint32_t) ((hr2 >> 1) & 1) << 31;
+    d.s64 = (uint32_t) hb2 << 31;
+    d.s128 = (uint32_t) hb3 << 31;
+    return d;
+}
+// stages with strides 16 .. 128 of a block of 256 floats held by the 16 lanes of a DPP row, 16 values per lane
+__device__ __forceinline__ void dpp_stages_256(float (&v)[16], const DppUnit &d) {
+    dpp_stage<0xB1>(v, d.s16);     // quad_perm [1, 0, 3, 2]
+    dpp_stage<0x4E>(v, d.s32);     // quad_perm [2, 3, 0, 1]
+    dpp_stage<0x141>(v, d.s64);    // row_half_mirror
+    dpp_stage<0x128>(v, d.s128);   // row_ror:8
+}
+
+// load_row_fwht16 for rows whose chunks are made of blocks of 256 floats (K is then a multiple of 256 and NT a multiple
+// of 64, so the 16 lanes of a DPP row are in or out of every round together): eight stages on the way in, four in
+// registers and four between lanes, and the row makes two trips through LDS less.
+template <int NT, int BATCH = 1>
+__device__ __forceinline__ void load_row_fwht256(float *buf, const float *__restrict__ xr, int K, int tid) {
+    const DppUnit d = dpp_unit_of_lane(tid & 63);
+    for (int u0 = tid; u0 < (K >> 4); u0 += NT * BATCH) {
+        float4 q[BATCH][4];
+#pragma unroll
+        for (int b = 0; b < BATCH; ++b) {
+            const int u = ((u0 + b * NT) & ~15) | d.unit;
+            if (u < (K >> 4)) {
+                const float4 *src = reinterpret_cast<const float4 *>(xr + 16 * u);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) q[b][j] = src[j];
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < BATCH; ++b) {
+            const int u = ((u0 + b * NT) & ~15) | d.unit;
+            if (u >= (K >> 4)) break;
+            float v[16] = { q[b][0].x, q[b][0].y, q[b][0].z, q[b][0].w, q[b][1].x, q[b][1].y, q[b][1].z, q[b][1].w,
+                            q[b][2].x, q[b][2].y, q[b][2].z, q[b][2].w, q[b][3].x, q[b][3].y, q[b][3].z, q[b][3].w };
+#pragma unroll
+            for (int h = 1; h < 16; h <<= 1) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    if ((j & h) == 0) {
+                        const float lo = v[j], up = v[j + h];
+                        v[j] = lo + up;
+                        v[j + h] = lo - up;
+                    }
+                }
+            }
+            dpp_stages_256(v, d);
+            float *dd = buf + padi(16 * u);
+#pragma unroll
+            for (int j = 0; j < 16; ++j) dd[j] = v[j];
+        }
+    }
+}
+
 // all Sylvester stages from stride 1 << ls0 up of every chunk of m = 1 << lm floats of a padded row, four stages per
 // trip through LDS
 __device__ __forceinline__ void fwht_row(float *buf, int K, int lm, int tid, int nt, int ls0 = 0) {

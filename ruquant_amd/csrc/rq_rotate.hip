@@ -46,10 +46,13 @@ __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs 
     const int wave = tid >> 6, lane = tid & 63;
 
     const float *xr = a.x + (int64_t) t * a.ldx;
-    // the first four Sylvester stages ride on the load (chunks here are multiples of 64)
-    load_row_fwht16<kRT>(buf, xr, K, tid);
+    // the first four Sylvester stages ride on the load (chunks here are multiples of 64), and the next four too,
+    // between lanes, when the chunks are made of blocks of 256 floats
+    const bool fused_256 = (m & 255) == 0;
+    if (fused_256) load_row_fwht256<kRT>(buf, xr, K, tid);
+    else load_row_fwht16<kRT>(buf, xr, K, tid);
     __syncthreads();
-    fwht_row(buf, K, lm, tid, kRT, 4);
+    fwht_row(buf, K, lm, tid, kRT, fused_256 ? 8 : 4);
 
     float *out = a.out_f32 + (int64_t) t * a.ldo;
     float *lh = a.lohi + (size_t) t * ng * 2;

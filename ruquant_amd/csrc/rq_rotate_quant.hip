@@ -27,11 +27,13 @@ constexpr int threads_of() { return SLICED && P < 44 ? 1024 : 512; }
 
 using namespace had;
 
-template <int P, bool SLICED>
+template <int P, bool SLICED, bool ALONE = false>
 // Registers are capped so that two workgroups (p >= 44: long columns, long rows) or three fit a compute unit: the
 // stages of one token are separated by barriers, and it is the other workgroups that keep the vector ALU busy. (The
-// sliced variant serves small batches, where occupancy is not the limit.)
-__global__ void __launch_bounds__((threads_of<P, SLICED>()), SLICED ? (P < 44 ? 4 : 2) : (P >= 44 ? 4 : 6))
+// sliced variant serves small batches, where occupancy is not the limit.) ALONE is the plain variant for rows so long
+// that LDS holds one workgroup per compute unit anyway: the cap then only makes the p >= 60 columns spill (136 to 504
+// bytes per lane), so it goes (2048 tokens, K = 26624, p = 104: 354 -> 269 us; K = 21504, p = 84: 204 -> 193 us).
+__global__ void __launch_bounds__((threads_of<P, SLICED>()), SLICED ? (P < 44 ? 4 : 2) : ALONE ? 2 : P >= 44 ? 4 : 6)
 rq_rotate_quant_kernel(const RotQuantArgs a) {
     constexpr int kNT = threads_of<P, SLICED>();
     extern __shared__ __align__(16) float smem[];
@@ -65,9 +67,15 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
     float *g_hi = g_lo + ng;
 
     const float *xr = a.x + (int64_t) t * a.ldx;
-    // the first four Sylvester stages ride on the load (one trip through LDS less per token)
+    // the first four Sylvester stages ride on the load (one trip through LDS less per token). In the sliced variant
+    // (small batches, bound by the latency of its phases) the next four ride too, between lanes, when the chunks are
+    // made of blocks of 256 floats; large batches are bound by vector-ALU time, where the LDS pass is the cheaper
+    // one (2048 tokens at K = 17408: 105 us against 128 us with the stages between lanes).
     const bool fused_first = a.rotate && (a.m & 15) == 0;
-    if (fused_first) {
+    const bool fused_256 = SLICED && a.rotate && (a.m & 255) == 0;
+    if (fused_256) {
+        load_row_fwht256<kNT, (P >= 44 ? 3 : 1)>(buf, xr, K, tid);
+    } else if (fused_first) {
         // long Paley stages go with long rows (several units of 16 floats per thread): all of a thread's loads go
         // out before the first butterfly
         load_row_fwht16<kNT, (P >= 44 ? 3 : 1)>(buf, xr, K, tid);
@@ -79,7 +87,7 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
     if (a.rotate) {
         const int m = a.m;
         const int lm = __ffs(m) - 1;
-        fwht_row(buf, K, lm, tid, kNT, fused_first ? 4 : 0);
+        fwht_row(buf, K, lm, tid, kNT, fused_256 ? 8 : fused_first ? 4 : 0);
         if constexpr (P > 1) {
             // Paley across the P chunks of every rotation block (reference lines 2466-2482), then the scale
             const int ncols = K / P;  // columns of all rotation blocks of this token
@@ -290,24 +298,29 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
 }
 
 // the kernels keep a whole row in dynamic LDS: raise the per-kernel limit (once per device, see init_activation_kernels)
-template <int P, bool SLICED>
+template <int P, bool SLICED, bool ALONE = false>
 hipError_t allow_big_lds() {
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_rotate_quant_kernel<P, SLICED>),
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_rotate_quant_kernel<P, SLICED, ALONE>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
 }
+
+// the plain variant has an ALONE build where the cap makes its columns spill and rows of up to RQ_MAX_K floats get that
+// long (p = 68 and 72 would need chunks of 512: past RQ_MAX_K)
+constexpr bool has_alone(int p) { return p == 60 || p >= 84; }
 
 template <int P>
 hipError_t allow_big_lds_both() {
     hipError_t e = allow_big_lds<P, false>();
     if (e == hipSuccess && P > 1) e = allow_big_lds<P, (P > 1)>();
+    if (e == hipSuccess && has_alone(P)) e = allow_big_lds<P, false, has_alone(P)>();
     return e;
 }
 
-template <int P, bool SLICED>
+template <int P, bool SLICED, bool ALONE = false>
 hipError_t launch_one(const RotQuantArgs &a, size_t lds, hipStream_t stream) {
     static bool attr_set = false;   // calls that never went through rq_w4a4_prepare on this device
     if (!attr_set) {
-        hipError_t e = allow_big_lds<P, SLICED>();
+        hipError_t e = allow_big_lds<P, SLICED, ALONE>();
         if (e != hipSuccess) return e;
         attr_set = true;
     }
@@ -317,7 +330,7 @@ hipError_t launch_one(const RotQuantArgs &a, size_t lds, hipStream_t stream) {
     b.token_blocks = a.M;
     const int grid = a.M + (int) ((a.zero_ints + (int64_t) kNT * 4 - 1) / ((int64_t) kNT * 4));
     if (grid == 0) return hipSuccess;
-    hipLaunchKernelGGL((rq_rotate_quant_kernel<P, SLICED>), dim3(grid), dim3(kNT), lds, stream, b);
+    hipLaunchKernelGGL((rq_rotate_quant_kernel<P, SLICED, ALONE>), dim3(grid), dim3(kNT), lds, stream, b);
     return hipGetLastError();
 }
 
@@ -331,6 +344,8 @@ hipError_t launch_p(const RotQuantArgs &a, hipStream_t stream) {
     if (P > 1 && a.M <= (P >= 44 ? kTwoStepTokens : 64) && 2 * row + stats <= 160 * 1024 - 64) {
         return launch_one<P, (P > 1)>(a, 2 * row + stats, stream);
     }
+    // a second workgroup does not fit beside this one
+    if (has_alone(P) && 2 * (row + stats + 64) > 160 * 1024) return launch_one<P, false, has_alone(P)>(a, row + stats, stream);
     return launch_one<P, false>(a, row + stats, stream);
 }
 

@@ -91,6 +91,21 @@ def test_quantizer_blocks_vs_oracle(oracle, K, had):
         assert got[t].tobytes() == want.tobytes(), "token %d" % t
 
 
+@pytest.mark.parametrize("K", [18432, 21504, 26624, 27648, 30720])
+def test_quantizer_long_rows_with_long_paley_stages(oracle, K):
+    """Rows of 72 x 256 (two workgroups still share a compute unit's LDS) and longer ones, where one leaves no room for
+    another (the build of the kernel without the register cap): Paley orders 84, 104, 108 and 60 (x 512)."""
+    rng = np.random.default_rng(K)
+    M = 3
+    x = (rng.standard_normal((M, K)) * np.exp2((np.arange(K) // 64 % 5 - 2))).astype(np.float32)
+    x[1, 1::3] = 0.0
+    clip = float(np.float32(0.85))
+    got = rq.quantize_act(torch.from_numpy(x).to(DEV), clip, hadamard_=True)
+    for t in range(M):
+        want = oracle.quantize_row_a4h(x[t], clip, K)
+        assert got[t].tobytes() == want.tobytes(), "token %d" % t
+
+
 # ---------------------------------------------------------------- MUL_MAT, the reference's test shapes
 
 def _shapes_reference():
@@ -162,6 +177,17 @@ def test_mul_mat_longest_row(oracle, type_, M):
     N, K = 128, 32768
     blocks, wf, W = _weights(oracle, N, K, type_)
     x = adversarial_activations(M, K, type_, wf, seed=3 * M)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=max(W.n_rot, 0))
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+@pytest.mark.parametrize("M", [2, 70])
+def test_mul_mat_long_row_long_paley_stage(oracle, M):
+    """K = 84 x 256: the activation kernel that has a compute unit to itself, feeding the GEMV and the GEMM."""
+    N, K, type_ = 136, 21504, rq.TYPE_W4A4H
+    blocks, wf, W = _weights(oracle, N, K, type_)
+    x = adversarial_activations(M, K, type_, wf, seed=5 * M)
     got = run_gpu(W, x)
     want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=max(W.n_rot, 0))
     assert bits_equal(got, want), first_mismatch(got, want)
