@@ -53,7 +53,7 @@ __global__ void __launch_bounds__(256) probe_stream_kernel(const v4u *__restrict
 // that the caller can check it).
 //   SAME  = true : every wavefront interleaves 1 MFMA with NV VALU instructions (roles ignored)
 //   SAME  = false: wavefronts 0..3 take role_lo, wavefronts 4..7 role_hi
-// OPK: 0 = v_add_u32, 1 = v_ashrrev_i32, 2 = v_mul_i32_i24
+// OPK: 0 = v_add_u32, 1 = v_ashrrev_i32, 2 = v_mul_i32_i24, 3 = v_dot8c_i32_i4 (eight chains of dependent ones)
 template <bool SAME, int NV, int OPK>
 __global__ void __launch_bounds__(512) probe_mix_kernel(int mfma_iters, int valu_iters, int role_lo, int role_hi,
                                                         int *sink, int *simd_of) {
@@ -74,11 +74,13 @@ __global__ void __launch_bounds__(512) probe_mix_kernel(int mfma_iters, int valu
                     if (OPK == 0) RQ_VALU8("v_add_u32");
                     if (OPK == 1) RQ_VALU8("v_ashrrev_i32");
                     if (OPK == 2) RQ_VALU8("v_mul_i32_i24");
+                    if (OPK == 3) RQ_VALU8("v_dot8c_i32_i4");
                 }
                 if (NV >= 16) {
                     if (OPK == 0) RQ_VALU8("v_add_u32");
                     if (OPK == 1) RQ_VALU8("v_ashrrev_i32");
                     if (OPK == 2) RQ_VALU8("v_mul_i32_i24");
+                    if (OPK == 3) RQ_VALU8("v_dot8c_i32_i4");
                 }
             }
         }
@@ -96,6 +98,7 @@ __global__ void __launch_bounds__(512) probe_mix_kernel(int mfma_iters, int valu
                     if (OPK == 0) RQ_VALU8("v_add_u32");
                     if (OPK == 1) RQ_VALU8("v_ashrrev_i32");
                     if (OPK == 2) RQ_VALU8("v_mul_i32_i24");
+                    if (OPK == 3) RQ_VALU8("v_dot8c_i32_i4");
                 }
             }
         }
@@ -185,6 +188,7 @@ extern "C" int rq_w4a4_probe(int kind, int64_t a0, int64_t a1, int64_t a2, int64
                 case 0: return (int) launch_mix<0>(sub, (int) a1, block, (int) a2, (int) a3, sink, simd_of, s);
                 case 1: return (int) launch_mix<1>(sub, (int) a1, block, (int) a2, (int) a3, sink, simd_of, s);
                 case 2: return (int) launch_mix<2>(sub, (int) a1, block, (int) a2, (int) a3, sink, simd_of, s);
+                case 3: return (int) launch_mix<3>(sub, (int) a1, block, (int) a2, (int) a3, sink, simd_of, s);
                 default: return RQ_E_ARGUMENT;
             }
         }

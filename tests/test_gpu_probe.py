@@ -23,7 +23,7 @@ def test_probe_kinds_launch_and_return():
         assert _probe(L, buf, STREAM, loads * 4096 * 16, loads, 0) == 0
     assert _probe(L, buf, STREAM, 1 << 22, 8, 64) == 0
     for sub in range(8):
-        for op in range(3):
+        for op in range(4):
             assert _probe(L, buf, MIX, sub | op << 8, 4, 2, 2) == 0
     assert _probe(L, buf, MIX, 5 | 1 << 16, 4, 2, 2) == 0
     assert _probe(L, buf, MIX, 0, 4, 2, 2) == 0
