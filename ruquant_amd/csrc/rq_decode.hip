@@ -133,10 +133,8 @@ __device__ __forceinline__ void quantize_rounds(const float *row, bool dense, in
 #pragma unroll
     for (int wr = 0; wr < R; ++wr) {
         const bool on = wr * kRotThreads + rt < nw;
-        float mn = fminf(fminf(fminf(fminf(0.0f, f[wr][0]), fminf(f[wr][1], f[wr][2])),
-                               fminf(fminf(f[wr][3], f[wr][4]), fminf(f[wr][5], f[wr][6]))), f[wr][7]);
-        float mx = fmaxf(fmaxf(fmaxf(fmaxf(0.0f, f[wr][0]), fmaxf(f[wr][1], f[wr][2])),
-                               fmaxf(fmaxf(f[wr][3], f[wr][4]), fmaxf(f[wr][5], f[wr][6]))), f[wr][7]);
+        float mn = 0.0f, mx = 0.0f;
+        minmax8_raw(f[wr], mn, mx);
         mn = group8_reduce<false>(mn);
         mx = group8_reduce<true>(mx);
         g_lo_r[wr] = mn * clip;

@@ -156,40 +156,62 @@ __device__ __forceinline__ void paley_column_generic(const float (&col)[P], floa
 // within quads, mirror the half rows, mirror the rows of 16, then carry across rows), which run at vector-ALU speed;
 // six dependent LDS-crossbar permutes would cost several hundred cycles each time, and the rotation kernels reduce
 // once per activation group.
+// Each step is ONE instruction, v_max_f32 / v_min_f32 with the permutation on its first operand, written as
+// assembly: from fmaxf(v, permuted v) the compiler makes four (a copy, the permutation as a move of its own, a
+// v_max_f32 x, x, x that quiets a signalling NaN, the max), because the language-level maximum is defined on quieted
+// operands. The instruction itself returns the other operand when one is a NaN, as fmaxf does. The s_nop in front is
+// the two wait states a DPP operand needs behind the vector instruction that wrote it (the compiler does not look
+// inside the assembly).
+#define RQ_DPP_MINMAX(v, ctrl)                                                                                   \
+    {                                                                                                            \
+        float r_;                                                                                                \
+        if (MAX) asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r_) : "v"(v)); \
+        else     asm("s_nop 1\n\tv_min_f32_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r_) : "v"(v)); \
+        v = r_;                                                                                                  \
+    }
+// (rows that the row mask leaves out keep their value: the operand is tied to the result)
+#define RQ_DPP_MINMAX_ROWS(v, ctrl, rows)                                                                        \
+    {                                                                                                            \
+        if (MAX) asm("s_nop 1\n\tv_max_f32_dpp %0, %0, %0 " ctrl " row_mask:" rows " bank_mask:0xf" : "+v"(v));   \
+        else     asm("s_nop 1\n\tv_min_f32_dpp %0, %0, %0 " ctrl " row_mask:" rows " bank_mask:0xf" : "+v"(v));   \
+    }
 template <bool MAX>
 __device__ __forceinline__ float wave_reduce(float v) {
-#define RQ_DPP_STEP(ctrl, row_mask)                                                                              \
-    {                                                                                                            \
-        const float o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v),         \
-                                                                              __builtin_bit_cast(int, v), ctrl,  \
-                                                                              row_mask, 0xF, false));            \
-        v = MAX ? fmaxf(v, o) : fminf(v, o);                                                                     \
-    }
-    RQ_DPP_STEP(0xB1, 0xF)    // quad_perm [1, 0, 3, 2]
-    RQ_DPP_STEP(0x4E, 0xF)    // quad_perm [2, 3, 0, 1]
-    RQ_DPP_STEP(0x141, 0xF)   // row_half_mirror
-    RQ_DPP_STEP(0x140, 0xF)   // row_mirror: every lane of a row now holds the row's value
-    RQ_DPP_STEP(0x142, 0xA)   // row_bcast:15 into rows 1 and 3
-    RQ_DPP_STEP(0x143, 0xC)   // row_bcast:31 into rows 2 and 3: lane 63 holds the wavefront's value
-#undef RQ_DPP_STEP
+    RQ_DPP_MINMAX(v, "quad_perm:[1,0,3,2]")
+    RQ_DPP_MINMAX(v, "quad_perm:[2,3,0,1]")
+    RQ_DPP_MINMAX(v, "row_half_mirror")
+    RQ_DPP_MINMAX(v, "row_mirror")                    // every lane of a row now holds the row's value
+    RQ_DPP_MINMAX_ROWS(v, "row_bcast:15", "0xa")      // into rows 1 and 3
+    RQ_DPP_MINMAX_ROWS(v, "row_bcast:31", "0xc")      // into rows 2 and 3: lane 63 holds the wavefront's value
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+// min / max of three as the one instruction, for operands that come straight from memory (the compiler would quiet
+// each of them first, an instruction per operand)
+__device__ __forceinline__ float min3_raw(float a, float b, float c) {
+    float r;
+    asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+// min(lo, v[0..7]) and max(hi, v[0..7])
+__device__ __forceinline__ void minmax8_raw(const float (&v)[8], float &lo, float &hi) {
+    lo = min3_raw(min3_raw(lo, v[0], v[1]), min3_raw(v[2], v[3], v[4]), min3_raw(v[5], v[6], v[7]));
+    hi = max3_raw(max3_raw(hi, v[0], v[1]), max3_raw(v[2], v[3], v[4]), max3_raw(v[5], v[6], v[7]));
 }
 // max / min over aligned runs of eight lanes, the same value in all eight
 template <bool MAX>
 __device__ __forceinline__ float group8_reduce(float v) {
-#define RQ_DPP_STEP(ctrl)                                                                                        \
-    {                                                                                                            \
-        const float o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v),         \
-                                                                              __builtin_bit_cast(int, v), ctrl,  \
-                                                                              0xF, 0xF, false));                 \
-        v = MAX ? fmaxf(v, o) : fminf(v, o);                                                                     \
-    }
-    RQ_DPP_STEP(0xB1)    // quad_perm [1, 0, 3, 2]
-    RQ_DPP_STEP(0x4E)    // quad_perm [2, 3, 0, 1]
-    RQ_DPP_STEP(0x141)   // row_half_mirror: lane i of a half row takes lane 7 - i, which sits in the other quad
-#undef RQ_DPP_STEP
+    RQ_DPP_MINMAX(v, "quad_perm:[1,0,3,2]")
+    RQ_DPP_MINMAX(v, "quad_perm:[2,3,0,1]")
+    RQ_DPP_MINMAX(v, "row_half_mirror")   // lane i of a half row takes lane 7 - i, which sits in the other quad
     return v;
 }
+#undef RQ_DPP_MINMAX
+#undef RQ_DPP_MINMAX_ROWS
 __device__ __forceinline__ float wave_max(float v) { return wave_reduce<true>(v); }
 __device__ __forceinline__ float wave_min(float v) { return wave_reduce<false>(v); }
 

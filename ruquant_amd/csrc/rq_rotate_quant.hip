@@ -172,10 +172,8 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
         float mn = 0.0f, mx = 0.0f;
         if (on) {
             const float *sp = buf + padi(8 * w);   // 8 consecutive values never straddle a run of 16
-            const float4 v0 = make_float4(sp[0], sp[1], sp[2], sp[3]);
-            const float4 v1 = make_float4(sp[4], sp[5], sp[6], sp[7]);
-            mn = fminf(fminf(fminf(fminf(mn, v0.x), fminf(v0.y, v0.z)), fminf(fminf(v0.w, v1.x), fminf(v1.y, v1.z))), v1.w);
-            mx = fmaxf(fmaxf(fmaxf(fmaxf(mx, v0.x), fmaxf(v0.y, v0.z)), fmaxf(fmaxf(v0.w, v1.x), fmaxf(v1.y, v1.z))), v1.w);
+            const float v8[8] = { sp[0], sp[1], sp[2], sp[3], sp[4], sp[5], sp[6], sp[7] };
+            had::minmax8_raw(v8, mn, mx);
         }
         if (lpg == 8) {
             // groups of 64 = eight lanes: swap within pairs, within quads, mirror the half row; DPP steps at vector-ALU
