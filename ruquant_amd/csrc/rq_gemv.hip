@@ -32,6 +32,14 @@ __device__ __forceinline__ int dot8(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot8((int) a, (int) b, c, false);
 }
 
+// a * b + c with a and b of at most 24 bits, as the one full-rate instruction (from __mul24(a, b) + c the compiler
+// makes a 64-bit multiply-add, which runs at a quarter of the rate)
+__device__ __forceinline__ int mad24(int a, int b, int c) {
+    int r;
+    asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
@@ -66,8 +74,10 @@ __device__ __forceinline__ void load_batch(Batch<U> &b, const uint4 *wp, int u0,
 
 // act: [run of 64 of the slice][token][8 words] codes q - 8 in the tensor's nibble order; mz: [unit of the slice][token]
 // m | (8 - z) << 8. The weight multiplier of a unit is that of its first run (reference patch line 168).
-template <int T, int kWaves, int U, int GF>
-__device__ __forceinline__ void compute_batch(const Batch<U> &b, const uint8_t *kp, bool hask, const uint32_t *act,
+// HASK (weight multipliers, a format variant) is a compile-time constant: as a run-time flag the compiler multiplies
+// every term by a multiplier that is 1, a full 32-bit multiply at a quarter of the rate.
+template <int T, int kWaves, int U, int GF, bool HASK>
+__device__ __forceinline__ void compute_batch(const Batch<U> &b, const uint8_t *kp, const uint32_t *act,
                                               const int32_t *mz, int u0, int u_begin, int u_end, int32_t (&tot)[T]) {
 #pragma unroll
     for (int j = 0; j < U / GF; ++j) {
@@ -100,15 +110,16 @@ __device__ __forceinline__ void compute_batch(const Batch<U> &b, const uint8_t *
                 acc = dot8(w[6], a1.z, acc);
                 acc = dot8(w[7], a1.w, acc);
                 const int zc = (int) (int8_t) ((mz[ul * T + t] >> 8) & 0xFF);
-                part[t] += acc + zc * cs;
+                part[t] += mad24(zc, cs, acc);   // |cs| <= 512, |zc| <= 8
             }
         }
         int kw = 1;
-        if (hask) kw = kp[(size_t) (u * GF) * kPanelRows];
+        if (HASK) kw = kp[(size_t) (u * GF) * kPanelRows];
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-            int term = (mz[ul * T + t] & 0xFF) * part[t];
-            if (hask) term *= kw;
+            // |part| <= 4 x 64 x 8 x 15 (an activation group of 256) and m <= 255: the 24-bit multiply is exact
+            int term = __mul24(mz[ul * T + t] & 0xFF, part[t]);
+            if (HASK) term *= kw;
             tot[t] += term >> kTermShift;
         }
     }
@@ -257,11 +268,19 @@ rq_gemv_kernel(const WeightSet ws, const float *__restrict__ x, int64_t ldx, con
     int32_t tot[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) tot[t] = 0;
-    compute_batch<T, kWaves, U, GF>(b0, kp, hask, s_act, s_mz, u_begin + wave, u_begin, u_end, tot);
+    if (hask) {
+        compute_batch<T, kWaves, U, GF, true>(b0, kp, s_act, s_mz, u_begin + wave, u_begin, u_end, tot);
+    } else {
+        compute_batch<T, kWaves, U, GF, false>(b0, kp, s_act, s_mz, u_begin + wave, u_begin, u_end, tot);
+    }
     for (int u0 = u_begin + wave + kWaves * (U / GF); u0 < u_end; u0 += kWaves * (U / GF)) {
         Batch<U> b;
         load_batch<kWaves, U, GF>(b, wp, u0, u_end);
-        compute_batch<T, kWaves, U, GF>(b, kp, hask, s_act, s_mz, u0, u_begin, u_end, tot);
+        if (hask) {
+            compute_batch<T, kWaves, U, GF, true>(b, kp, s_act, s_mz, u0, u_begin, u_end, tot);
+        } else {
+            compute_batch<T, kWaves, U, GF, false>(b, kp, s_act, s_mz, u0, u_begin, u_end, tot);
+        }
     }
 
 #pragma unroll
