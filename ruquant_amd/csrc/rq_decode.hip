@@ -73,6 +73,19 @@ __device__ __forceinline__ int dot8(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot8((int) a, (int) b, c, false);
 }
 
+// a * b + c with a and b of at most 24 bits as the one full-rate instruction (from __mul24(a, b) + c the compiler
+// makes a 64-bit multiply-add, which runs at a quarter of the rate); the first form takes `a` from a scalar register
+__device__ __forceinline__ int mad24_s(int a, int b, int c) {
+    int r;
+    asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "s"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ int mad24(int a, int b, int c) {
+    int r;
+    asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 __device__ __forceinline__ int align4(int v) { return (v + 3) & ~3; }
 
 // Barrier among the rotate wavefronts only, through a counter in LDS that only grows: a wavefront adds one when its
@@ -386,7 +399,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                         cs = dot8(w[j][1].z, 0x11111111u, cs);
                         cs = dot8(w[j][1].w, 0x11111111u, cs);
                         // |acc|, |cs * (8 - z)| <= 4096 and m <= 255: 24-bit multiplies are exact
-                        const int part = acc + __mul24((int) (int8_t) ((mzv >> 8) & 0xFF), cs);
+                        const int part = mad24_s((int) (int8_t) ((mzv >> 8) & 0xFF), cs, acc);
                         int term = __mul24(on ? (mzv & 0xFF) : 0, part);
                         if (fl & 1) term *= (int) kmul[((size_t) wpanel * ng + g) * kPanelRows + lane];
                         tot += term >> kTermShift;
@@ -432,7 +445,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                     cs = dot8(wt[it].y, 0x11111111u, cs);
                     cs = dot8(wt[it].z, 0x11111111u, cs);
                     cs = dot8(wt[it].w, 0x11111111u, cs);
-                    int part = acc + __mul24((int) (int8_t) ((mzv >> 8) & 0xFF), cs);
+                    int part = mad24((int) (int8_t) ((mzv >> 8) & 0xFF), cs, acc);
                     // the other half of the group sits eight lanes away in the same row of 16 lanes
                     part += __builtin_amdgcn_update_dpp(0, part, 0x128 /* row_ror:8 */, 0xF, 0xF, false);
                     int term = __mul24(mzv & 0xFF, part);
