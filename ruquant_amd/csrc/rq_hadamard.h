@@ -162,19 +162,14 @@ __device__ __forceinline__ void paley_column_generic(const float (&col)[P], floa
 // operands. The instruction itself returns the other operand when one is a NaN, as fmaxf does. The s_nop in front is
 // the two wait states a DPP operand needs behind the vector instruction that wrote it (the compiler does not look
 // inside the assembly).
-#define RQ_DPP_MINMAX(v, ctrl)                                                                                   \
-    {                                                                                                            \
-        float r_;                                                                                                \
-        if (MAX) asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r_) : "v"(v)); \
-        else     asm("s_nop 1\n\tv_min_f32_dpp %0, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf" : "=v"(r_) : "v"(v)); \
-        v = r_;                                                                                                  \
-    }
-// (rows that the row mask leaves out keep their value: the operand is tied to the result)
+// The operand is tied to the result: a lane whose partner is switched off, and the rows that a row mask leaves out,
+// keep their value.
 #define RQ_DPP_MINMAX_ROWS(v, ctrl, rows)                                                                        \
     {                                                                                                            \
         if (MAX) asm("s_nop 1\n\tv_max_f32_dpp %0, %0, %0 " ctrl " row_mask:" rows " bank_mask:0xf" : "+v"(v));   \
         else     asm("s_nop 1\n\tv_min_f32_dpp %0, %0, %0 " ctrl " row_mask:" rows " bank_mask:0xf" : "+v"(v));   \
     }
+#define RQ_DPP_MINMAX(v, ctrl) RQ_DPP_MINMAX_ROWS(v, ctrl, "0xf")
 template <bool MAX>
 __device__ __forceinline__ float wave_reduce(float v) {
     RQ_DPP_MINMAX(v, "quad_perm:[1,0,3,2]")
