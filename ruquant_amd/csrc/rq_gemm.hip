@@ -99,6 +99,15 @@ __device__ __forceinline__ void load_to_lds(const uint4 *gptr, uint4 *lds) {
                  : "memory", "m0");
 }
 
+// 64 lanes x 4 bytes to 256 bytes of LDS
+__device__ __forceinline__ void load_to_lds_dword(const float *gptr, float *lds) {
+    const uint32_t lds_addr = (uint32_t) (uintptr_t) (lds_void *) lds;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+                 :
+                 :  "v"(gptr), "s"(lds_addr)
+                 : "memory", "m0");
+}
+
 // fetch of step `st` into stage s: every wavefront moves three 1 KiB runs. Groups past the end are clamped to the
 // last one (refetched into cells nobody reads).
 template <int MODE>
@@ -388,6 +397,10 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     __shared__ Stage s3;
     __shared__ Stage s4;
     __shared__ Stage s5;
+    // the epilogue's operands, fetched with the first groups: the scales of the tile's 256 rows, then the units of its
+    // tokens (at the end of the tile, their trip from memory, two microseconds, would stand between the last group
+    // and the stores)
+    __shared__ __align__(16) float s_pre[256 + kBT];
     constexpr bool NARROW = MODE == kNarrow;
     constexpr int TT = tiles_of(MODE);
     constexpr int kTok = MODE == kHalf ? kBTh : kBT;   // tokens of a wide or half tile
@@ -467,6 +480,16 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
         }
     }
 
+    {
+        const int lane = tid & 63;
+        if (c.wave < 4) {
+            const int64_t n = (int64_t) panel0 * kPanelRows + 64 * c.wave + lane;
+            load_to_lds_dword(s_w + (n < N ? n : N - 1), &s_pre[64 * c.wave]);
+        } else if (c.wave < 6) {
+            const int t = t0 + 64 * (c.wave - 4) + lane;
+            load_to_lds_dword(u + (t < M ? t : M - 1), &s_pre[256 + 64 * (c.wave - 4)]);
+        }
+    }
     if (flags[0] & 1) {
         gemm_body<true, MODE>(c, s0, s1, s2, s3, s4, s5, k_src, hi, lo);
     } else {
@@ -517,13 +540,13 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
     for (int ct = 0; ct < TT; ++ct) {
         const int t = t0 + (NARROW ? 0 : MODE == kHalf ? 32 * c.wc : 64 * c.wc) + 16 * ct + c.l16;
         if (t >= M) continue;
-        const float ut = u[t];
+        const float ut = s_pre[256 + (t - t0)];
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) {
             const int64_t n = (int64_t) (panel0 + c.wr) * kPanelRows + 16 * rt + 4 * c.quad;
             float *dst = y + (int64_t) t * ldy + n;
+            const float4 sw = *reinterpret_cast<const float4 *>(&s_pre[64 * c.wr + 16 * rt + 4 * c.quad]);
             if (n + 3 < N && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
-                const float4 sw = *reinterpret_cast<const float4 *>(s_w + n);
                 float4 o;
                 o.x = (((float) tot[rt][ct][0] * 16.0f) * ut) * sw.x;
                 o.y = (((float) tot[rt][ct][1] * 16.0f) * ut) * sw.y;
@@ -534,9 +557,10 @@ rq_gemm_kernel(const uint4 *__restrict__ codes, const float *__restrict__ s_w, c
                 typedef float v4f __attribute__((ext_vector_type(4)));
                 __builtin_nontemporal_store(v4f{ o.x, o.y, o.z, o.w }, reinterpret_cast<v4f *>(dst));
             } else {
+                const float swv[4] = { sw.x, sw.y, sw.z, sw.w };
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    if (n + i < N) dst[i] = (((float) tot[rt][ct][i] * 16.0f) * ut) * s_w[n + i];
+                    if (n + i < N) dst[i] = (((float) tot[rt][ct][i] * 16.0f) * ut) * swv[i];
                 }
             }
         }
