@@ -28,13 +28,13 @@
 #ifdef RQ_DECODE_TIMING
 // Phase timestamps of workgroup 0 (wavefronts 0 and 8), kept in registers and written out at the very end: a store in
 // the middle of the kernel would queue behind the weight stream and distort what it measures.
-__device__ unsigned long long rq_decode_stamps[64];
-#define RQ_STAMP_DECL unsigned long long rq_st[8] = {}
+__device__ unsigned long long rq_decode_stamps[64];   // [0, 16) rotate wavefront, [32, 48) stream wavefront
+#define RQ_STAMP_DECL unsigned long long rq_st[16] = {}
 #define RQ_STAMP(i) do { rq_st[(i)] = __builtin_readcyclecounter(); } while (0)
 #define RQ_STAMP_AT(st, i) do { (st)[(i)] = __builtin_readcyclecounter(); } while (0)
 #define RQ_STAMP_PTR rq_st
 #define RQ_STAMP_FLUSH do { if (blockIdx.x == 0 && (threadIdx.x == 0 || threadIdx.x == 512)) { \
-        for (int i_ = 0; i_ < 8; ++i_) rq_decode_stamps[i_ + (threadIdx.x ? 32 : 0)] = rq_st[i_]; } } while (0)
+        for (int i_ = 0; i_ < 16; ++i_) rq_decode_stamps[i_ + (threadIdx.x ? 32 : 0)] = rq_st[i_]; } } while (0)
 extern "C" int rq_w4a4_decode_stamps(unsigned long long *out) {
     return (int) hipMemcpyFromSymbol(out, HIP_SYMBOL(rq_decode_stamps), sizeof(rq_decode_stamps));
 }
@@ -103,11 +103,17 @@ __device__ __forceinline__ void wait_count(const int *cnt, int target) {
     }
     asm volatile("" ::: "memory");
 }
+// (The add needs no wait for the wavefront's LDS writes in front of it: a wavefront's LDS instructions are carried out in
+// the order of issue, so whoever sees the count sees the writes. It returns the count, and the wavefront that
+// arrives last, the one the others wait for, knows so from the answer and does not poll: two LDS round trips less on
+// the critical path of every phase.)
 __device__ __forceinline__ void rot_sync(int *cnt, int &target, int lane) {
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (lane == 0) atomicAdd(cnt, 1);
     target += kRotWaves;
-    wait_count<false>(cnt, target);
+    int seen = 0;
+    if (lane == 0) seen = atomicAdd(cnt, 1) + 1;
+    seen = __builtin_amdgcn_readfirstlane(seen);
+    if (seen < target) wait_count<false>(cnt, target);
+    asm volatile("" ::: "memory");
 }
 
 // The activation quantizer of the rotate wavefronts for R code words per thread (word w = r x 512 + thread, its eight
@@ -142,6 +148,10 @@ __device__ __forceinline__ void quantize_rounds(const float *row, bool dense, in
             for (int j = 0; j < 8; ++j) f[wr][j] = 0.0f;
         }
     }
+#ifdef RQ_DECODE_TIMING
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // (the values have arrived from LDS)
+#endif
+    RQ_STAMP_AT(stamps, 10);
     float rmax = 0.0f;
 #pragma unroll
     for (int wr = 0; wr < R; ++wr) {
@@ -156,6 +166,7 @@ __device__ __forceinline__ void quantize_rounds(const float *row, bool dense, in
     }
     rmax = wave_max(rmax);
     if (lane == 0) s_part[wave] = rmax;
+    RQ_STAMP_AT(stamps, 11);
     rot_sync(s_cnt, sync_target, lane);
     RQ_STAMP_AT(stamps, 5);
 
@@ -183,6 +194,7 @@ __device__ __forceinline__ void quantize_rounds(const float *row, bool dense, in
             if ((w & 7) == 0) s_mz[w >> 3] = mg | ((8 - (int) zf) & 0xFF) << 8;
         }
     }
+    RQ_STAMP_AT(stamps, 12);
 }
 
 // LDS: [row, padded][Paley output, dense][codes][mz][cells][wave maxima, unit, phase counter]
@@ -506,6 +518,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                 for (int j = 0; j < 16; ++j) d[j] = v[j];
             }
         }
+        RQ_STAMP(8);
         rot_sync(s_cnt, sync_target, lane);
         RQ_STAMP(2);
 
@@ -584,6 +597,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
 #pragma unroll
                     for (int o = 0; o < kOut; ++o) dst[o * m] = out[o] * a.scale;
                 }
+                RQ_STAMP(9);
                 rot_sync(s_cnt, sync_target, lane);
             } else {
                 for (int i = rt; i < K; i += kRotThreads) buf[padi(i)] = buf[padi(i)] * a.scale;

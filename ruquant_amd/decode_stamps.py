@@ -34,13 +34,21 @@ def main():
         for _ in range(3):
             rq.mul_mat(W, x)
             torch.cuda.synchronize()
-        out = (ctypes.c_ulonglong * 64)()
+        out = (ctypes.c_ulonglong * 64)()   # [0, 16) rotate wavefront, [32, 48) stream wavefront
         if L.rq_w4a4_decode_stamps(out) != 0:
             raise RuntimeError("rq_w4a4_decode_stamps failed")
         st = list(out)
         print("K=%d N=%d (cycles since the rotate wavefront entered the kernel)" % (K, N))
         for i, name in enumerate(ROTATE):
             print("  rotate wavefront  %-28s %7d" % (name, st[i] - st[0]))
+        # the same wavefront, in front of the wait at the end of each stage: what a stage computes and what it waits
+        for name, before, after in (("row written to LDS", 8, 2), ("Paley sums written", 9, 4),
+                                    ("group ranges computed", 11, 5), ("codes written", 12, 6)):
+            if st[before]:
+                print("  rotate wavefront  %-28s %7d  (then %d until every rotate wavefront has)"
+                      % (name, st[before] - st[0], st[after] - st[before]))
+        if st[10]:
+            print("  rotate wavefront  %-28s %7d" % ("values of the ranges read", st[10] - st[0]))
         for i, name in enumerate(STREAM):
             print("  stream wavefront  %-28s %7d" % (name, st[32 + i] - st[0]))
         sys.stdout.flush()
