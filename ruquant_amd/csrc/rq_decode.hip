@@ -259,6 +259,31 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
     // 11.0, and a barrier held the stream back until the row had arrived. With the row first, that barrier only
     // cost time: 8.5 -> 7.7 us at N = 5120.)
     __builtin_amdgcn_s_barrier();
+    RQ_STAMP(13);
+
+    // ---- The stream wavefronts request the first round of their first whole panel here, in front of everything else
+    // they work out (rows and cells, the remainder's addresses: 1700 cycles). The barrier above is what keeps the
+    // token's row in front of them in the memory pipeline: the rotate wavefronts ask for it before they arrive there.
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    v4u w[MG > 0 ? MG : 1][2];
+    constexpr int kEarly = MG < 4 ? MG : 4;   // groups asked for here (their registers are live through all that follows)
+    if constexpr (MG > 0) {
+        if (wave >= kRotWaves) {
+            const int sw = wave - kRotWaves;
+            const int panel = blockIdx.x;   // the first of panels s, s + G, ...
+            const int wsel = (panel >= a.ws.first[1]) + (panel >= a.ws.first[2]);
+            const int wpanel = panel - (wsel == 0 ? 0 : wsel == 1 ? a.ws.first[1] : a.ws.first[2]);
+            const uint8_t *codes = wsel == 0 ? a.ws.codes[0] : wsel == 1 ? a.ws.codes[1] : a.ws.codes[2];
+            const uint8_t *pbase = codes + (size_t) wpanel * ng * 2048 + lane * 16;
+#pragma unroll
+            for (int j = 0; j < kEarly; ++j) {
+                int g = sw + j * kStrWaves;
+                if (g >= ng) g = 0;   // past the end: the first group again, contributes nothing
+                w[j][0] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(pbase + (size_t) g * 2048));
+                w[j][1] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(pbase + (size_t) g * 2048 + 1024));
+            }
+        }
+    }
 
     // ---- this workgroup's rows: whole panels s, s + G, ..., and a run of quads of the remainder panels. Remainder
     // slots run over the XCDs so that slots t and t + 1 (which may share an octet) sit on one XCD: workgroups go to
@@ -302,6 +327,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         }
     }
 
+    RQ_STAMP(14);
     if (wave >= kRotWaves) {
         // =========================================================== the weight stream
         const int sw = wave - kRotWaves;
@@ -317,7 +343,6 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         const bool anyk = ((f0 | f1 | f2) & 1) != 0;
         const int n_items = n_oct * nblk;
         const int codes_ready = kRotWaves * (1 + a.n_pass + (a.rotate ? 1 : 0) + 2);
-        typedef unsigned v4u __attribute__((ext_vector_type(4)));
         bool waited = false;
 
         // remainder item `i` of this workgroup -> address of its 1 KiB (8 rows x 4 groups x 2 halves)
@@ -343,6 +368,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
             }
         }
 
+        RQ_STAMP(15);
         // ---- whole panels: lane = row, a group is two 1 KiB loads; the wavefront takes groups sw, sw + 8, ...
         if constexpr (MG > 0) {
             const int gpw = (ng + kStrWaves - 1) / kStrWaves;   // groups per wavefront and panel
@@ -356,9 +382,11 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                 const uint8_t *pbase = codes + (size_t) wpanel * ng * 2048 + lane * 16;
                 int tot = 0;
                 for (int gi0 = 0; gi0 < gpw; gi0 += MG) {
-                    v4u w[MG][2];
+                    // (the first groups of the first panel's first round are in flight since the kernel's start)
+                    const bool first = pl == 0 && gi0 == 0;
 #pragma unroll
                     for (int j = 0; j < MG; ++j) {
+                        if (j < kEarly && first) continue;
                         int g = sw + (gi0 + j) * kStrWaves;
                         if (g >= ng) g = 0;   // past the end: the first group again, contributes nothing
                         w[j][0] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(pbase + (size_t) g * 2048));

@@ -51,6 +51,9 @@ def main():
             print("  rotate wavefront  %-28s %7d" % ("values of the ranges read", st[10] - st[0]))
         for i, name in enumerate(STREAM):
             print("  stream wavefront  %-28s %7d" % (name, st[32 + i] - st[0]))
+        for name, i in (("first barrier passed", 13), ("rows and cells worked out", 14), ("remainder items requested", 15)):
+            if st[32 + i]:
+                print("  stream wavefront  %-28s %7d" % (name, st[32 + i] - st[0]))
         sys.stdout.flush()
 
 
