@@ -266,7 +266,11 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
     // token's row in front of them in the memory pipeline: the rotate wavefronts ask for it before they arrive there.
     typedef unsigned v4u __attribute__((ext_vector_type(4)));
     v4u w[MG > 0 ? MG : 1][2];
-    constexpr int kEarly = MG < 4 ? MG : 4;   // groups asked for here (their registers are live through all that follows)
+    // groups asked for here: their registers are live through all that follows. 2 take 0.03 us off the headline
+    // call, 4 take 0.2, 6 take 0.24, 8 no longer fit the registers (+0.5 us). The 12-group form that also carries
+    // remainder items has no register to spare: with any asked for early it spills more (K = 6144, N = 17408:
+    // 13.6 -> 14.8 us).
+    constexpr int kEarly = (MG >= 12 && MT > 0) ? 0 : MG < 6 ? MG : 6;
     if constexpr (MG > 0) {
         if (wave >= kRotWaves) {
             const int sw = wave - kRotWaves;
