@@ -19,7 +19,10 @@ using namespace had;
 
 constexpr int kRT = 512;  // threads per workgroup
 
-template <int P>
+// O = outputs of a column that one Paley item (one wavefront) forms: four, or two for a long stage and few tokens
+// (twice the workgroups, half the chain of additions per wavefront: 6.9 -> 6.5 us for one token of K = 17408; at 16
+// tokens the workgroups would no longer be resident together: 10.2 -> 11.5 us)
+template <int P, int O>
 __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs a, int slabs, int parts) {
     extern __shared__ __align__(16) float buf[];
     __shared__ float s_rmax[kRT / 64];
@@ -44,6 +47,7 @@ __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs 
     const int K = a.K, m = a.m, ng = K / kGroup;
     const int lm = __ffs(m) - 1;
     const int wave = tid >> 6, lane = tid & 63;
+    constexpr int kO = O;
 
     const float *xr = a.x + (int64_t) t * a.ldx;
     // the first four Sylvester stages ride on the load (chunks here are multiples of 64), and the next four too,
@@ -75,20 +79,19 @@ __global__ void __launch_bounds__(kRT) rq_rotate_slab_kernel(const RotQuantArgs 
     } else {
         // wave-items = (rotation block, slice of four output chunks) for this slab's 64 columns
         const int n_rb = K / a.n_rot;
-        const int n_items = n_rb * (P / 4);
+        const int n_items = n_rb * (P / kO);
         const int pm = m + (m >> 4);
         for (int wi = part + parts * wave; wi < n_items; wi += parts * (kRT / 64)) {
             const int s = wi / n_rb, rb = wi - s * n_rb;
             const int b0 = rb * a.n_rot + 64 * slab + lane;
             const float *src = buf + padi(b0);
-            float col[P];
+            // (the four sums advance together, one column element at a time: four independent chains of dependent
+            // additions; one sum after the other the wavefront waits out every addition's latency)
+            float res[kO];
+            paley_pick_stream<P, kO, 0>(s, src, pm, res);
 #pragma unroll
-            for (int i = 0; i < P; ++i) col[i] = src[i * pm];
-            float res[4];
-            paley_pick<P, 4>(s, col, res);
-#pragma unroll
-            for (int o = 0; o < 4; ++o) {
-                const int idx = b0 + (4 * s + o) * m;
+            for (int o = 0; o < kO; ++o) {
+                const int idx = b0 + (kO * s + o) * m;
                 const float v = res[o] * a.scale;
                 out[idx] = v;
                 const float lo = wave_min(fminf(v, 0.0f)) * a.clip, hi = wave_max(fmaxf(v, 0.0f)) * a.clip;
@@ -151,42 +154,76 @@ __global__ void __launch_bounds__(kRT) rq_quantize_digits_kernel(const RotQuantA
     *reinterpret_cast<uint2 *>(dst + (size_t) 16 * a.Mp) = make_uint2(hi_e, hi_o);
 }
 
-template <int P>
+template <int P, int O>
 hipError_t allow_big_lds() {
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_rotate_slab_kernel<P>),
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&rq_rotate_slab_kernel<P, O>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
+}
+
+// the two-output form exists for the long Paley stage only
+constexpr bool has_pairs(int p) { return p > 44; }
+
+template <int P>
+hipError_t allow_big_lds_p() {
+    hipError_t e = allow_big_lds<P, 4>();
+    if constexpr (has_pairs(P)) {
+        if (e == hipSuccess) e = allow_big_lds<P, 2>();
+    }
+    return e;
+}
+
+// workgroups per token that share a slab's Paley items: enough that a wavefront gets one item, within the token's
+// range slots
+inline int parts_of(int n_items, int slabs) {
+    int parts = (n_items + kRT / 64 - 1) / (kRT / 64);
+    while (parts > 1 && slabs * parts > kRangeParts) --parts;
+    return parts;
 }
 
 template <int P>
 hipError_t launch_slab(const RotQuantArgs &a, hipStream_t stream) {
     static bool attr_set = false;   // calls that never went through rq_w4a4_prepare on this device
     if (!attr_set) {
-        hipError_t e = allow_big_lds<P>();
+        hipError_t e = allow_big_lds_p<P>();
         if (e != hipSuccess) return e;
         attr_set = true;
     }
     // one slab per 64 columns of a chunk; without a Paley stage, a few workgroups share the row's runs
     int slabs = P > 1 ? a.m / 64 : (a.K >= 4096 ? 4 : 1);
-    // enough parts that a wavefront gets one Paley item, within the token's range slots
-    const int n_items = P > 1 ? (a.K / a.n_rot) * (P / 4) : 0;
-    int parts = P > 1 ? (n_items + kRT / 64 - 1) / (kRT / 64) : 1;
     if (slabs > kRangeParts) return launch_rotate_quant(a, stream);   // more slabs than range slots
-    while (parts > 1 && slabs * parts > kRangeParts) --parts;
+    const int n_rb = a.K / a.n_rot;
+    int parts = P > 1 ? parts_of(n_rb * (P / 4), slabs) : 1;
+    bool pairs = false;
+    if constexpr (has_pairs(P)) {
+        // items of two outputs while all the workgroups are still resident together (one per compute unit)
+        const int parts2 = parts_of(n_rb * (P / 2), slabs);
+        if (a.M * slabs * parts2 <= 256) {
+            pairs = true;
+            parts = parts2;
+        }
+    }
     const int zero_blocks = (int) ((a.zero_ints + (int64_t) kRT * 4 - 1) / ((int64_t) kRT * 4));
     RotQuantArgs b = a;
     b.token_blocks = a.M * slabs * parts;
     const size_t lds = (size_t) (a.K + (a.K >> 4) + 1) * sizeof(float);
-    hipLaunchKernelGGL((rq_rotate_slab_kernel<P>), dim3(b.token_blocks + zero_blocks), dim3(kRT), lds, stream, b, slabs, parts);
+    const dim3 grid(b.token_blocks + zero_blocks);
+    if constexpr (has_pairs(P)) {
+        if (pairs) {
+            hipLaunchKernelGGL((rq_rotate_slab_kernel<P, 2>), grid, dim3(kRT), lds, stream, b, slabs, parts);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((rq_rotate_slab_kernel<P, 4>), grid, dim3(kRT), lds, stream, b, slabs, parts);
     return hipGetLastError();
 }
 
 }  // namespace
 
 hipError_t init_rotate_slab_kernels() {
-    hipError_t e = allow_big_lds<1>();
-    if (e == hipSuccess) e = allow_big_lds<12>();
-    if (e == hipSuccess) e = allow_big_lds<20>();
-    if (e == hipSuccess) e = allow_big_lds<68>();
+    hipError_t e = allow_big_lds_p<1>();
+    if (e == hipSuccess) e = allow_big_lds_p<12>();
+    if (e == hipSuccess) e = allow_big_lds_p<20>();
+    if (e == hipSuccess) e = allow_big_lds_p<68>();
     return e;
 }
 
