@@ -379,7 +379,7 @@ def test_config3_prefill_gemm(oracle, M):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
-@pytest.mark.parametrize("M", [1, 16, 2048])
+@pytest.mark.parametrize("M", [1, 12, 13, 16, 2048])   # (12 / 13: the rotation goes from items of two outputs to four)
 def test_config4_down_projection(oracle, M):
     K, N = 17408, 5120
     blocks = synth.random_weight_blocks(N, K, 4, rq.TYPE_W4A4H)
