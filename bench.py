@@ -38,11 +38,14 @@ INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA
 HEADLINE_PROFILE = os.path.join(ROOT, "profiles", "decode_m1_k5120_n17408.md")
 
 
-def profiled_traffic_bytes(path=HEADLINE_PROFILE):
+GEMM_PROFILE = os.path.join(ROOT, "profiles", "gemm_m2048.md")   # "traffic_bytes_per_launch_m2048: <n>", both launches
+
+
+def profiled_traffic_bytes(path=HEADLINE_PROFILE, key="traffic_bytes_per_launch:"):
     try:
         with open(path) as f:
             for line in f:
-                if line.startswith("traffic_bytes_per_launch:"):
+                if line.startswith(key):
                     return int(line.split(":")[1].split()[0])
     except OSError:
         pass
@@ -461,7 +464,8 @@ def main():
             if name == "prefill_k5120_n17408_m2048":
                 ops = 2.0 * m * n * k
                 roofline_m2048 = {"bound": "mfma", "achieved": round(ops / kms / 1e9, 1), "peak": INT8_PEAK_TOPS,
-                                  "unit": "TOP/s", "frac": round(ops / kms / 1e9 / INT8_PEAK_TOPS, 4), "traffic": None,
+                                  "unit": "TOP/s", "frac": round(ops / kms / 1e9 / INT8_PEAK_TOPS, 4),
+                                  "traffic": profiled_traffic_bytes(GEMM_PROFILE, "traffic_bytes_per_launch_m2048:"),
                                   "kernel": "rq_gemm_kernel (wide + narrow tiles of one launch)",
                                   "kernel_us": round(kms * 1e3, 3), "workload": "W4A4H K=5120 N=17408 M=2048",
                                   "op_us": extra[name]["op_us"], "op_tops": extra[name]["op_tops"],
