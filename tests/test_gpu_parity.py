@@ -379,6 +379,43 @@ def test_config3_prefill_gemm(oracle, M):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
+@pytest.mark.parametrize("type_,K,N,n_rot,mult", [
+    (rq.TYPE_W4A4H, 5120, 17408, 5120, 0),     # the headline: one whole panel per workgroup and a quad of the remainder
+    (rq.TYPE_W4A4H, 5120, 17408, 5120, 256),   # ... with a weight multiplier per block
+    (rq.TYPE_W4A4H, 5120, 17408, 5120, 64),    # ... per group of 64
+    (rq.TYPE_W4A4H, 5120, 16384, 5120, 0),     # whole panels only
+    (rq.TYPE_W4A4H, 5120, 33216, 5120, 0),     # two whole panels per workgroup, 7 remainder panels
+    (rq.TYPE_W4A4H, 6144, 16576, 6144, 0),     # 12 groups per stream wavefront with remainder items (H12 x H512)
+    (rq.TYPE_W4A4H, 6144, 16576, 6144, 64),
+    (rq.TYPE_W4A4H, 6144, 16384, 6144, 0),     # 12 groups, no remainder
+    (rq.TYPE_W4A4H, 10240, 16448, 10240, 0),   # two rounds of 10 groups per panel (H20 x H512)
+    (rq.TYPE_W4A4H, 12288, 16448, 12288, 256), # two rounds of 12 groups (H12 x H1024)
+    (rq.TYPE_W4A4H, 8192, 16640, 8192, 0),     # 16 groups per wavefront: 12 + 4 and clamped loads, no Paley stage
+    (rq.TYPE_W4A4H, 16384, 16448, 16384, 0),   # the longest row the kernel takes: 32 groups per wavefront, three rounds
+    (rq.TYPE_W4A4H, 5120, 16448, 2560, 0),     # block-diagonal rotation (H20 x H128 twice)
+    (rq.TYPE_W4A4, 4096, 16448, 0, 0),         # no rotation: 8 groups per wavefront in a round of 10
+    (rq.TYPE_W4A4, 6144, 17408, 0, 64),
+])
+def test_one_token_whole_panels(oracle, type_, K, N, n_rot, mult):
+    """One token against weights of at least 256 panels of 64 rows, where every workgroup of the one-launch kernel
+    streams whole panels (its stream wavefronts hold 10 or 12 groups per round, the first ones requested before
+    anything else) beside its share of the remainder. `mult`: integer weight multipliers in the block headers, one
+    per block of 256 codes or one per group of 64 (reference patch lines 38-43)."""
+    had = type_ == rq.TYPE_W4A4H
+    blocks = synth.random_weight_blocks(N, K, 11, type_, clip=0.9, n_rot=n_rot if had else None)
+    rng = np.random.default_rng(13)
+    if mult == 256:
+        blocks["sum"] = ((1 << 30) | rng.integers(1, 16, size=blocks["sum"].shape)).astype(np.int32)
+    elif mult == 64:
+        k = rng.integers(1, 16, size=blocks["sum"].shape + (4,))
+        blocks["sum"] = ((3 << 29) | k[..., 0] | (k[..., 1] << 4) | (k[..., 2] << 8) | (k[..., 3] << 12)).astype(np.int32)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    x = synth.activations("outlier_channels", 1, K, 12)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=n_rot if had else 0)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
 @pytest.mark.parametrize("M", [1, 12, 13, 16, 2048])   # (12 / 13: the rotation goes from items of two outputs to four)
 def test_config4_down_projection(oracle, M):
     K, N = 17408, 5120
