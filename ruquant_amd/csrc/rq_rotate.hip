@@ -197,7 +197,7 @@ hipError_t launch_slab(const RotQuantArgs &a, hipStream_t stream) {
     if constexpr (has_pairs(P)) {
         // items of two outputs while all the workgroups are still resident together (one per compute unit)
         const int parts2 = parts_of(n_rb * (P / 2), slabs);
-        if (a.M * slabs * parts2 <= 256) {
+        if (a.M * slabs * parts2 <= device_compute_units()) {
             pairs = true;
             parts = parts2;
         }
