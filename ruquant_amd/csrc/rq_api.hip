@@ -112,10 +112,13 @@ bool rotation_of(int type, int64_t K, int64_t n_rot, int &p, int &m) {
     return hadamard_factor(n_rot, p, m);
 }
 
-// Measured crossovers (K = 5120, N = 17408): up to three tokens the dot-product GEMV, from four the skinny MFMA
-// kernel, from 65 the tiled MFMA GEMM.
+// Measured crossovers: up to four tokens the dot-product GEMV, from five the skinny MFMA kernel, from 65 the tiled
+// MFMA GEMM. (Four tokens, K = 5120, whole call on the GEMV against the skinny kernel: N = 1024 9.1 against 11.4 us,
+// N = 5120 11.8 against 12.3, N = 8192 and 17408 the same, N = 34816 26.2 against 25.5: the GEMV's activation side is
+// one launch, the skinny kernel's two. Five tokens: 13.7 against 12.3 us at N = 5120, 22.7 against 18.0 at N = 17408.
+// The choice depends on the token count only, so that a quantized activation can be shared between weights.)
 enum Path { kPathGemv, kPathSkinny, kPathGemm };
-constexpr int kGemvMax = 3;
+constexpr int kGemvMax = 4;
 Path path_of(int64_t M) {
     if (M > kSkinnyTokens) return kPathGemm;
     return M <= kGemvMax ? kPathGemv : kPathSkinny;

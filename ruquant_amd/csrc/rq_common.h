@@ -18,7 +18,7 @@ constexpr int kRangeParts = 32;    // partial maxima of a token's group ranges h
 constexpr int kSkinnyTokens = 64;   // most tokens of one pass of the skinny MFMA kernel
 constexpr int kTwoStepTokens = 40;   // long Paley stages: most tokens whose rotation is spread over several workgroups each
 constexpr int kGemvWideTokens = 8;   // most tokens of a GEMV pass with activation groups of 128 / 256
-constexpr int kGemvMaxTokens = 64;  // workspaces of up to this many tokens hold the fp32 form too (the GEMV takes up to 3
+constexpr int kGemvMaxTokens = 64;  // workspaces of up to this many tokens hold the fp32 form too (the GEMV takes up to 4
                                     // tokens, up to 8 with activation groups of 128 / 256; the skinny path's two-step
                                     // activation side uses the fp32 rows as an intermediate)
 
@@ -66,7 +66,7 @@ inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
 // Workspace of one rq_w4a4_mul_mat call.
 //
 //   u      : Mp floats, the token units (GEMM path; the GEMV derives them itself).
-//   act    : GEMV path (M <= 3; M <= 8 with wide activation groups): the rotated activations as fp32 rows [M][K] followed by the clipped group
+//   act    : GEMV path (M <= 4; M <= 8 with wide activation groups): the rotated activations as fp32 rows [M][K] followed by the clipped group
 //            ranges [M][ng][2] (lo, hi) and [M][32] partial maxima of hi - lo; every GEMV workgroup quantizes
 //            the K slice it consumes itself.
 //            MFMA paths: two int8 digit planes of m (q - z), [g][digit][quarter][Mp][16 bytes], in the byte order
