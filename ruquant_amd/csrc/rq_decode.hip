@@ -204,6 +204,28 @@ __host__ __device__ inline size_t decode_lds_bytes(int K, bool two_rows) {
     return (size_t) (Kp + (two_rows ? K : 0) + K / 8 + ng + kDecodeCells + 8 + kRotWaves + 4) * 4;
 }
 
+// Two Paley items of one wavefront, column runs `cr` and `cr + 1` of slice `s` (a run = 64 neighbouring columns, a
+// slice = P / 4 of a column's outputs), as one instruction stream: from the padded row `buf` to the dense row `alt`.
+template <int P>
+__device__ __forceinline__ void paley_pair(const float *buf, float *alt, int s, int cr, int lane, int lm, int m,
+                                           int n_rot, int pm, float scale) {
+    constexpr int kOut = P / 4;
+    const int c0 = cr * 64 + lane, c1 = c0 + 64;
+    const int b0 = (c0 >> lm) * n_rot + (c0 & (m - 1)), b1 = (c1 >> lm) * n_rot + (c1 & (m - 1));
+    float out0[kOut], out1[kOut];
+    if (m == 256) {
+        paley_pick_stream2<P, kOut, 272>(s, buf + padi(b0), buf + padi(b1), 272, out0, out1);
+    } else {
+        paley_pick_stream2<P, kOut, 0>(s, buf + padi(b0), buf + padi(b1), pm, out0, out1);
+    }
+    float *d0 = alt + b0 + kOut * s * m, *d1 = alt + b1 + kOut * s * m;
+#pragma unroll
+    for (int o = 0; o < kOut; ++o) {
+        d0[o * m] = out0[o] * scale;
+        d1[o * m] = out1[o] * scale;
+    }
+}
+
 // MG: group-items (64 rows x one group: two loads) a stream wavefront has in flight per round of a whole panel;
 // MT: remainder items (8 rows x 4 groups: one load) per round. The first round of both is issued up front.
 template <int P, int MG, int MT>
@@ -583,26 +605,24 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                 const int per_wave = (n_it + kRotWaves - 1) / kRotWaves;
                 if (per_wave == 2 && (col_runs & 1) == 0 && (ncols & 63) == 0 && 2 * wave + 1 < n_it) {
                     // the wavefront's two items are neighbouring column runs of one slice: one instruction stream
-                    // for both (whole row rotated as H20 x H256 or H12 x H512: 16 items for eight wavefronts)
+                    // for both (whole row rotated as H20 x H256 or H12 x H256: 16 items for eight wavefronts)
                     int s = 0, cr = 2 * wave;
                     while (cr >= col_runs) {
                         cr -= col_runs;
                         ++s;
                     }
-                    const int c0 = cr * 64 + lane, c1 = c0 + 64;
-                    const int b0 = (c0 >> lm) * a.n_rot + (c0 & (m - 1)), b1 = (c1 >> lm) * a.n_rot + (c1 & (m - 1));
-                    float out0[kOut], out1[kOut];
-                    if (m == 256) {
-                        paley_pick_stream2<P, kOut, 272>(s, buf + padi(b0), buf + padi(b1), 272, out0, out1);
-                    } else {
-                        paley_pick_stream2<P, kOut, 0>(s, buf + padi(b0), buf + padi(b1), pm, out0, out1);
+                    paley_pair<P>(buf, alt, s, cr, lane, lm, m, a.n_rot, pm, a.scale);
+                } else if ((per_wave & 1) == 0 && col_runs % per_wave == 0 && (ncols & 63) == 0 &&
+                           per_wave * (wave + 1) <= n_it) {
+                    // four or eight items per wavefront (H12 x H512, H20 x H512: 32 items; H12 x H1024: 64): they are
+                    // neighbouring column runs of one slice as well, taken two at a time (one at a time, K = 6144:
+                    // 9.5 us for the call at N = 5120 against 8.9 us; four at a time: 8.8 us)
+                    int s = 0, cr = per_wave * wave;
+                    while (cr >= col_runs) {
+                        cr -= col_runs;
+                        ++s;
                     }
-                    float *d0 = alt + b0 + kOut * s * m, *d1 = alt + b1 + kOut * s * m;
-#pragma unroll
-                    for (int o = 0; o < kOut; ++o) {
-                        d0[o * m] = out0[o] * a.scale;
-                        d1[o * m] = out1[o] * a.scale;
-                    }
+                    for (int pr = 0; pr < per_wave; pr += 2) paley_pair<P>(buf, alt, s, cr + pr, lane, lm, m, a.n_rot, pm, a.scale);
                 } else
                 for (int it = 0; it < per_wave; ++it) {
                     const int wi = wave * per_wave + it;
