@@ -46,8 +46,10 @@ namespace {
 struct Env {
     float clip[2];   // RQ_ACT_CLIP, RQ_ACT_CLIP_H (falls back to the former); -1 = unset
     int   act_group;
-    int   decode_fused;   // one token: the single-launch kernel. RQ_DECODE_FUSED=0 (the one debug switch of the
-                          // library) sends one token down the rotation kernel + GEMV that serves two and three
+    int   decode_fused;   // one token: the single-launch kernel. RQ_DECODE_FUSED=0 (a debug switch) sends one token
+                          // down the rotation kernel + GEMV that serves two and three
+    int   gemm_fp6;       // wide batches: the fp6 MFMA kernel on the weight's fp6 plane. RQ_GEMM_FP6=0 leaves the plane
+                          // out of prepared weights (0.75 bytes per weight) and runs the int8 MFMA kernel instead
     Env() {
         const char *e = getenv("RQ_ACT_CLIP");
         const char *eh = getenv("RQ_ACT_CLIP_H");
@@ -58,6 +60,8 @@ struct Env {
         act_group = v == 128 || v == 256 ? v : 64;
         const char *df = getenv("RQ_DECODE_FUSED");
         decode_fused = df ? atoi(df) != 0 : 1;
+        const char *f6 = getenv("RQ_GEMM_FP6");
+        gemm_fp6 = f6 ? atoi(f6) != 0 : 1;
     }
 };
 
@@ -65,6 +69,12 @@ const Env &env() {
     static const Env e;
     return e;
 }
+
+}  // namespace
+
+bool gemm_fp6_enabled() { return env().gemm_fp6 != 0; }
+
+namespace {
 
 // Device address of `scratch` on the current device, resolved once per device (each GPU holds its own copy of the
 // array at its own address). Returns null with *err set when the runtime refuses.
@@ -218,7 +228,9 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     // the skinny path: one plane of q - z and the multipliers beside it (half the activation bytes per group, which
     // count against the weight bytes a compute unit can have in flight)
     const bool single = path == kPathSkinny;
-    q.single = single;
+    const bool fp6 = path == kPathGemm && gemm_fp6_enabled();
+    q.single = fp6 ? 2 : single;
+    q.m4 = reinterpret_cast<float *>(wsb + W.off_i8 + act6_plane_bytes((int) (K / kGroup), W.Mp));
     q.mvals = reinterpret_cast<uint8_t *>(wsb + W.off_i8) + (size_t) (K / kGroup) * act_mp * 64;
     const float *gemv_x = x;      // what the GEMV quantizes from: the rotated rows, or x itself for W4A4
     int64_t gemv_ldx = ldx;
@@ -291,7 +303,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             g.M = (int) M;
             g.Mp = (int) W.Mp;
             g.groups_per_fold = G / kGroup;
-            e = launch_gemm(g, stream);
+            e = fp6 ? launch_gemm6(g, stream) : launch_gemm(g, stream);
             if (e != hipSuccess) return (int) e;
         } else {
             for (int c = 0; c < W.chunks; ++c) {

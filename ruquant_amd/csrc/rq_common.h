@@ -33,13 +33,26 @@ constexpr int kGemvMaxTokens = 64;  // workspaces of up to this many tokens hold
 //   s_w   : n_panels x 64 floats (rows past N are zero).
 //   kmul  : n_panels x ng x 64 bytes, the integer weight multiplier of (row, group): 1 for legacy headers.
 //   flags : one int32; bit 0 set when any multiplier differs from 1 (kernels branch on it, uniformly).
+//   w6    : (unless RQ_GEMM_FP6=0) the same codes once more as fp6 (E2M3) MFMA fragments for wide token batches:
+//           n_rtiles x ng x 8 fragments x 1536 bytes. Fragment f of row tile R (rows 256 R + 32 f ..), group g:
+//           lane l = row % 32 + 32 * half holds inputs 64 g + 32 half .. + 31 as 32 six-bit values (sign, then the
+//           magnitude 0 .. 8: as fp6 the value is code / 8), value j in bits 6j .. 6j+5 of the lane's 24 bytes; bytes
+//           0 .. 15 of lane l sit at l * 16, bytes 16 .. 23 at 1024 + l * 8. Rows past N are zero.
 // ---------------------------------------------------------------------------------------------------
+constexpr int kFrag6 = 1536;      // bytes of one 32 x 64 fp6 MFMA fragment
+constexpr int kRowTile6 = 256;    // rows of one tile of the fp6 plane
+
 struct PreparedLayout {
     int64_t K, N;
     int     ng;        // K / 64
     int     n_panels;  // ceil(N / 64)
-    size_t  off_codes, off_sw, off_kmul, off_flags, bytes;
+    int     n_rtiles;  // ceil(N / 256)
+    size_t  off_codes, off_sw, off_kmul, off_flags, off_w6, bytes;   // off_w6 == 0: no fp6 plane
 };
+
+// whether prepared weights carry the fp6 plane and wide batches use the fp6 MFMA kernel (RQ_GEMM_FP6, default on;
+// read once per process)
+bool gemm_fp6_enabled();
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -49,6 +62,7 @@ inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
     L.N = N;
     L.ng = (int) (K / kGroup);
     L.n_panels = (int) ((N + kPanelRows - 1) / kPanelRows);
+    L.n_rtiles = (int) ((N + kRowTile6 - 1) / kRowTile6);
     size_t off = 0;
     L.off_codes = off;
     off = align_up(off + (size_t) L.n_panels * L.ng * 2048, 256);
@@ -58,9 +72,17 @@ inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
     off = align_up(off + (size_t) L.n_panels * L.ng * kPanelRows, 256);
     L.off_flags = off;
     off = align_up(off + 256, 256);
+    L.off_w6 = 0;
+    if (gemm_fp6_enabled()) {
+        L.off_w6 = off;
+        off = align_up(off + (size_t) L.n_rtiles * L.ng * 8 * kFrag6, 256);
+    }
     L.bytes = off;
     return L;
 }
+
+// bytes of the fp6 activation plane of Mp tokens (a multiple of 32); the multipliers follow it as [ng][Mp] floats
+inline size_t act6_plane_bytes(int ng, int64_t Mp) { return (size_t) ng * (size_t) (Mp / 32) * kFrag6; }
 
 // ---------------------------------------------------------------------------------------------------
 // Workspace of one rq_w4a4_mul_mat call.
@@ -71,7 +93,9 @@ inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
 //            the K slice it consumes itself.
 //            MFMA paths: two int8 digit planes of m (q - z), [g][digit][quarter][Mp][16 bytes], in the byte order
 //            the weight unpack produces (for M <= 64 they follow the fp32 form, which the skinny path may use as
-//            an intermediate).
+//            an intermediate). The fp6 GEMM (M >= 65) takes one plane of q - z as fp6 MFMA fragments instead,
+//            [g][Mp / 32][1536 bytes] (lane = token % 32 + 32 * half, as in the weight plane), followed by the
+//            group multipliers as floats 4 m, [g][Mp].
 //   cells  : split-K cells [8 or 64 tokens][n_panels * 64], 64 bits each: arrival count above bit 48, exact sum
 //            below.
 // ---------------------------------------------------------------------------------------------------
@@ -136,10 +160,12 @@ struct RotQuantArgs {
     int32_t      len_field;               // kActBlocks: pad[1] of the activation blocks (K or n_rot)
     float       *u;
     uint32_t    *act;                     // kActI8
-    // kActI8, single-plane form for the skinny kernel: one int8 plane of q - z
-    // [g][quarter][Mp][16 bytes] at `act`, and the group multipliers m as bytes [g][Mp] at `mvals`
+    // kActI8, single-plane form for the skinny kernel (single == 1): one int8 plane of q - z
+    // [g][quarter][Mp][16 bytes] at `act`, and the group multipliers m as bytes [g][Mp] at `mvals`.
+    // single == 2: the fp6 fragment plane of q - z at `act` and the multipliers as floats 4 m, [g][Mp], at `m4`
     int          single;
     uint8_t     *mvals;
+    float       *m4;
     int          Mp;                      // kActI8: padded token count (rows M..Mp-1 are zero filled)
     // split-K scratch to clear (blocks past the token blocks do it)
     int32_t     *zero_ptr;
@@ -227,6 +253,8 @@ struct GemmArgs {
     int             groups_per_fold;   // 1; 2 or 4 when the activation groups are 128 or 256 wide
 };
 hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
+// the fp6 form: act8 = the fp6 fragment plane with the multipliers behind it; the weight needs the fp6 plane
+hipError_t launch_gemm6(const GemmArgs &a, hipStream_t stream);
 
 // up to 64 tokens: MFMA arithmetic on a GEMV-shaped weight stream; same operands as the GEMM plus the split-K cells
 struct SkinnyArgs {

@@ -1,0 +1,440 @@
+// int4 x int4 GEMM for wide token batches on the gfx950 matrix cores, through v_mfma_f32_32x32x64_f8f6f4 with fp6
+// (E2M3) operands: the MFMA form that runs at twice the rate of the int8 one and whose K = 64 is exactly one
+// activation group.
+//
+// Why fp6 is exact here. An E2M3 value with sign s and the five exponent / mantissa bits read as the integer n
+// (0 .. 31) is n / 8 for n <= 15 (subnormals 0 .. 7 / 8, then 1 .. 1.875 in steps of 1 / 8): the sign-magnitude code
+// of an integer |v| <= 15 IS the fp6 encoding of v / 8. Weight codes w (-8 .. 7) and activation values q - z
+// (-15 .. 15) both fit, every product w (q - z) / 64 is a multiple of 1 / 64 below 2, and a group's sum
+// S / 64 (|S| <= 7680) is exact in the fp32 accumulator. One MFMA per 32 x 32 outputs and group yields
+// S_g = sum_k w_k (q_k - z_g), which equals the reference's acc + (8 - z) colsum (ggml_vec_dot_w4a4_a4, reference
+// patch lines 160-172).
+//
+// The per-group floor. The reference adds floor(m_g S_g / 16) per group (reference patch lines 35-39, 173). With the
+// wavefront's fp32 rounding mode set toward minus infinity, acc = fma(S / 64, 4 m, acc) on an accumulator that
+// holds an integer in [2^23, 2^24) (where one unit in the last place is 1) is acc + floor(m S / 16): the FMA forms
+// m S / 16 + acc exactly and rounds once, downwards, to an integer. One full-rate vector instruction per output and
+// group. The accumulator starts at 1.5 x 2^23; a group moves it by at most 255 x 7680 / 16 = 122,400, so after 32
+// groups (3,916,800 < 2^22) its offset from the start is moved into an int32 total (two integer instructions per
+// value: the float's bit pattern minus the bit pattern of 1.5 x 2^23 is that offset) and it starts again.
+//
+// Tensors with integer weight multipliers k (uniform branch on the prepared flag) fold
+// floor(k m S / 16) in integers instead. Activation groups of 128 / 256 (RQ_ACT_GROUP) chain the 2 or 4 MFMAs of a
+// group through the accumulator operand before the one fold.
+//
+// Data movement: a workgroup of eight wavefronts owns 256 rows x 128 tokens; wavefront (wr, wc) owns rows 64 wr .. and
+// tokens 64 wc .. as 2 x 2 MFMA tiles of 32 x 32. Operands go from global memory straight into LDS
+// (global_load_lds_dwordx4), two groups per ring stage, four stages. Both the fp6 weight plane that
+// rq_w4a4_prepare writes and the activation plane of the quantizer are stored as MFMA fragments (32 rows or tokens x
+// 64 inputs = 1536 bytes: a 16-byte and an 8-byte piece per lane, each piece contiguous across the lanes), so a
+// stage is filled by whole 1 KiB runs and read back without bank conflicts.
+#include "rq_common.h"
+
+#include <string.h>
+
+#pragma clang fp contract(off)
+
+namespace rq {
+
+namespace {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void lds_void;
+
+constexpr int kThreads = 512;
+constexpr int kTileRows = 256;                 // rows of a workgroup's tile
+constexpr int kTileTok = 128;                  // tokens of a workgroup's tile
+constexpr int kCellsA = 8 * kFrag6 / 16;       // 768 cells: eight weight fragments of one group
+constexpr int kCellsB = 4 * kFrag6 / 16;       // 384 cells: four activation fragments of one group
+constexpr int kCellsM = kTileTok * 4 / 16;     // 32 cells: the 128 tokens' multipliers of one group (4 m as float)
+// One ring stage = two groups: [A g0][A g1][B g0][B g1][m g0][m g1] = 2368 cells of 16 bytes = 37 KiB
+constexpr int kOffA = 0, kOffB = 2 * kCellsA, kOffM = kOffB + 2 * kCellsB;
+constexpr int kStageCells = kOffM + 2 * kCellsM;
+constexpr int kRing = 4;
+static_assert(kStageCells == 2368, "stage size");
+// Each wavefront moves four whole 1 KiB runs per step (cells 0 .. 2047: the weights and the first 512 activation
+// cells) and 40 lanes' worth of a fifth (cells 2048 .. 2367: the rest of the activations and the multipliers).
+constexpr int kTailCell = 2048, kTailLanes = 40;
+static_assert(kTailCell + 8 * kTailLanes == kStageCells, "tail split");
+constexpr int kLoadsPerStep = 5;
+
+constexpr float kBias = 12582912.0f;           // 1.5 x 2^23
+constexpr int kBiasBits = 0x4B400000;
+constexpr int kFlushSteps = 16;                // 32 groups
+
+struct Stage {
+    uint4 cell[kStageCells];
+};
+
+// 64 lanes x 16 bytes from base + lane offset to 1 KiB of LDS at `lds` (wave-uniform; the hardware adds lane * 16).
+// Assembly, so that the count of outstanding loads stays under this file's control (the s_waitcnt of step()).
+// a wave-uniform address, said so explicitly: the compiler then keeps it in scalar registers
+__device__ __forceinline__ const uint8_t *uniform(const uint8_t *p) {
+    const uint64_t b = (uint64_t) (uintptr_t) p;
+    return reinterpret_cast<const uint8_t *>(
+        (uintptr_t) ((uint64_t) (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) b) |
+                     (uint64_t) (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (b >> 32)) << 32));
+}
+
+__device__ __forceinline__ void load_run(const uint8_t *base, uint32_t lane_off, uint4 *lds) {
+    const uint32_t lds_addr = (uint32_t) (uintptr_t) (lds_void *) lds;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_off), "s"(base), "s"(lds_addr)
+                 : "memory", "m0");
+}
+
+// the same from per-lane addresses, for the lanes of `mask` only (the others move nothing). The execution mask is
+// switched inside the statement: a branch around the load would cut the step into several basic blocks, and the
+// compiler then sinks the folds of one step behind the barrier of the next (their inputs, 128 registers, spill).
+__device__ __forceinline__ void load_cells(const uint8_t *gptr, uint4 *lds, uint64_t mask) {
+    const uint32_t lds_addr = (uint32_t) (uintptr_t) (lds_void *) lds;
+    uint64_t saved;
+    asm volatile("s_mov_b32 m0, %2\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, %3\n\t"
+                 "global_load_lds_dwordx4 %1, off\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved)
+                 : "v"(gptr), "s"(lds_addr), "s"(mask)
+                 : "memory", "m0");
+}
+
+__device__ __forceinline__ void load_to_lds_dword(const float *gptr, float *lds) {
+    const uint32_t lds_addr = (uint32_t) (uintptr_t) (lds_void *) lds;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+                 :
+                 : "v"(gptr), "s"(lds_addr)
+                 : "memory", "m0");
+}
+
+struct Ctx {
+    // the four whole runs this wavefront moves per step: address of step 0 and advance per step (wave-uniform)
+    const uint8_t *run_src[4];
+    size_t run_step[4];
+    const uint8_t *tail_src; // this lane's cell of the fifth load, current step
+    size_t tail_step;        // its advance per step
+    const uint8_t *k_src;    // weight multipliers of this wavefront's panel, row offset of the lane's first quad
+    int wave, wr, wc, lane;
+    int n_steps;
+};
+
+// fetch of the next step (two groups) into stage s, then advance the sources; past the last step they stay where they
+// are (the last step is fetched again, into cells nobody reads), so every step issues the same number of loads
+__device__ __forceinline__ void fetch(Ctx &c, Stage &s, int st) {
+    const uint32_t lane_off = (uint32_t) c.lane * 16;
+    const bool more = st + 1 < c.n_steps;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        load_run(c.run_src[i], lane_off, &s.cell[(i * 8 + c.wave) * 64]);
+        c.run_src[i] = uniform(c.run_src[i] + (more ? c.run_step[i] : 0));
+    }
+    load_cells(c.tail_src, &s.cell[kTailCell + c.wave * kTailLanes], ((uint64_t) 1 << kTailLanes) - 1);
+    c.tail_src += more ? c.tail_step : 0;
+}
+
+__device__ __forceinline__ v8i fragment(const Stage &s, int cell0, int lane) {
+    const uint4 p0 = s.cell[cell0 + lane];
+    const uint2 p1 = *(reinterpret_cast<const uint2 *>(&s.cell[cell0 + 64]) + lane);
+    v8i v;
+    v[0] = (int) p0.x; v[1] = (int) p0.y; v[2] = (int) p0.z; v[3] = (int) p0.w;
+    v[4] = (int) p1.x; v[5] = (int) p1.y;
+    // (the fp6 form reads six registers: elements 6 and 7 are left undefined)
+    return v;
+}
+
+// fast path: acc += floor(m S / 16) for the 16 outputs of one tile (round toward minus infinity is set)
+__device__ __forceinline__ void fold_fast(const v16f &S, float m4, float (&acc)[16]) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = __builtin_fmaf(S[r], m4, acc[r]);
+}
+
+// weight multipliers: tot += floor(k m S / 16) in integers (reference patch line 173)
+__device__ __forceinline__ void fold_k(const v16f &S, float m4, const int (&kk)[16], int32_t (&tot)[16]) {
+    const int mi = (int) (m4 * 0.25f);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int Si = (int) (S[r] * 64.0f);
+        tot[r] += (kk[r] * mi * Si) >> kTermShift;
+    }
+}
+
+// One step (two groups of 64 inputs) of one wavefront: 64 rows x 64 tokens as 2 x 2 tiles. GS = runs of 64 per
+// activation group (1, 2, 4). A unit = one tile x one activation group's runs inside this step: its MFMAs chain through
+// the accumulator operand; the fold of unit i runs behind the MFMAs of unit i + 1.
+template <bool HASK, int GS>
+__device__ __forceinline__ void compute(const Ctx &c, const Stage &s, int st, float (&acc)[2][2][16],
+                                        int32_t (&tot)[2][2][16], v16f (&carry)[2][2]) {
+    constexpr int kRuns = GS == 1 ? 1 : 2;        // runs of a unit inside one step
+    constexpr int kUnits = GS == 1 ? 8 : 4;
+    v8i A[2][2], B[2][2];
+    float m4[2][2];
+#pragma unroll
+    for (int gi = 0; gi < 2; ++gi) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            A[gi][i] = fragment(s, kOffA + gi * kCellsA + (2 * c.wr + i) * (kFrag6 / 16), c.lane);
+            B[gi][i] = fragment(s, kOffB + gi * kCellsB + (2 * c.wc + i) * (kFrag6 / 16), c.lane);
+            m4[gi][i] = reinterpret_cast<const float *>(&s.cell[kOffM + gi * kCellsM])[64 * c.wc + 32 * i + (c.lane & 31)];
+        }
+    }
+    // with groups of 256 a unit spans two steps: the even step leaves its half in `carry`, the odd step folds
+    const bool folds = GS < 4 || (st & 1);
+    const bool starts = GS < 4 || !(st & 1);
+    const v16f zero = {};
+    v16f S[2];
+    int prev_a = 0, prev_b = 0, prev_gi = 0;
+#pragma unroll
+    for (int un = 0; un < kUnits + 1; ++un) {
+        if (un < kUnits) {
+            const int gi = GS == 1 ? un >> 2 : 0, a = (un >> 1) & 1, b = un & 1;
+            v16f C = GS == 4 && !starts ? carry[a][b] : zero;
+#pragma unroll
+            for (int run = 0; run < kRuns; ++run) {
+                C = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[gi + run][a], B[gi + run][b], C, 2, 2, 0, 0, 0, 0);
+            }
+            if (GS == 4 && !folds) carry[a][b] = C;
+            S[un & 1] = C;
+        }
+        if (un > 0 && folds) {
+            const v16f &P = S[(un - 1) & 1];
+            if (!HASK) {
+                fold_fast(P, m4[prev_gi][prev_b], acc[prev_a][prev_b]);
+            } else {
+                // the multiplier of the group's first run (reference patch line 171: RQ_W_MULT_G(sum, sg << (2 - lsub)))
+                const int g = (GS == 4 ? 2 * (st & ~1) : 2 * st) + prev_gi;
+                int k16[16];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t k4 = *reinterpret_cast<const uint32_t *>(c.k_src + (size_t) g * kPanelRows + 32 * prev_a + 8 * q);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) k16[4 * q + i] = (k4 >> (8 * i)) & 0xFF;
+                }
+                fold_k(P, m4[prev_gi][prev_b], k16, tot[prev_a][prev_b]);
+            }
+        }
+        if (un < kUnits) {
+            prev_gi = GS == 1 ? un >> 2 : 0;
+            prev_a = (un >> 1) & 1;
+            prev_b = un & 1;
+        }
+        // a unit's MFMAs and the previous unit's fold stay together: left alone, the scheduler issues all the
+        // (independent) MFMAs of a step first, and their results (16 registers each) spill
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+template <bool HASK, int GS>
+__device__ __forceinline__ void step(Ctx &c, const Stage &cur, Stage &refill, int st, float (&acc)[2][2][16],
+                                     int32_t (&tot)[2][2][16], v16f (&carry)[2][2]) {
+    // the loads of steps st + 1 and st + 2 may still be in flight
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerStep) : "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    fetch(c, refill, st + 3);
+    compute<HASK, GS>(c, cur, st, acc, tot, carry);
+}
+
+__device__ __forceinline__ void flush(float (&acc)[2][2][16], int32_t (&tot)[2][2][16]) {
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                tot[a][b][r] += __builtin_bit_cast(int, acc[a][b][r]) - kBiasBits;
+                acc[a][b][r] = kBias;
+            }
+        }
+    }
+}
+
+template <bool HASK, int GS>
+__device__ __forceinline__ void body(Ctx &c, Stage &s0, Stage &s1, Stage &s2, Stage &s3,
+                                     float (&acc)[2][2][16], int32_t (&tot)[2][2][16]) {
+    v16f carry[2][2] = {};
+    fetch(c, s0, 0);
+    fetch(c, s1, 1);
+    fetch(c, s2, 2);
+    for (int st = 0; st < c.n_steps; st += kRing) {
+        // (K is a multiple of 256: the number of steps is even, so steps come in pairs)
+        step<HASK, GS>(c, s0, s3, st, acc, tot, carry);
+        step<HASK, GS>(c, s1, s0, st + 1, acc, tot, carry);
+        if (st + 2 < c.n_steps) {
+            step<HASK, GS>(c, s2, s1, st + 2, acc, tot, carry);
+            step<HASK, GS>(c, s3, s2, st + 3, acc, tot, carry);
+        }
+        if (!HASK && ((st / kRing + 1) % (kFlushSteps / kRing)) == 0) flush(acc, tot);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the refetches of the last steps
+}
+
+template <int GS>
+__global__ void __launch_bounds__(kThreads)
+rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
+                const int32_t *__restrict__ flags, const uint8_t *__restrict__ act6, const float *__restrict__ m4,
+                const float *__restrict__ u, float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng,
+                int n_panels, int n_tok_tiles, int n_tiles, int super_tiles) {
+    __shared__ Stage s0;
+    __shared__ Stage s1;
+    __shared__ Stage s2;
+    __shared__ Stage s3;
+    // the epilogue's operands, fetched ahead of the first groups: the scales of the tile's 256 rows, then the units of
+    // its 128 tokens
+    __shared__ __align__(16) float s_pre[kTileRows + kTileTok];
+
+    // Workgroups go to the eight XCDs round robin: every XCD gets a contiguous run of tiles, visited in super-tiles of
+    // 8 row tiles x 4 token tiles (the 32 workgroups an XCD runs at a time then share 8 weight tiles and 4 activation
+    // tiles in its L2), or with the token tiles running fastest where the launch is not made of whole super-tiles.
+    int row_tile, t0;
+    {
+        int v = blockIdx.x;
+        const int per_xcd = n_tiles / kXcds;
+        if (v < per_xcd * kXcds) v = (v % kXcds) * per_xcd + v / kXcds;
+        if (super_tiles) {
+            const int s = v >> 5, i = v & 31;
+            const int spr = n_tok_tiles >> 2;
+            const int sr = s / spr;
+            row_tile = sr * 8 + (i >> 2);
+            t0 = ((s - sr * spr) * 4 + (i & 3)) * kTileTok;
+        } else {
+            row_tile = v / n_tok_tiles;
+            t0 = (v - row_tile * n_tok_tiles) * kTileTok;
+        }
+    }
+    const int tid = threadIdx.x;
+    Ctx c;
+    c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    c.wr = c.wave & 3;
+    c.wc = c.wave >> 2;
+    c.lane = tid & 63;
+    c.n_steps = ng / 2;
+    const uint8_t *w_tile = w6 + (size_t) row_tile * ng * (kCellsA * 16);   // this tile's rows, group 0
+    const size_t a_step = (size_t) (Mp / 32) * kFrag6;                       // bytes between groups of the activation plane
+    const uint8_t *a_tile = act6 + (size_t) (t0 / 32) * kFrag6;              // this tile's tokens, group 0
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        // run L of the stage: runs 0 .. 23 are the weights of the step's two groups (12 each), 24 .. 35 the activations
+        // (6 each; the last four belong to the fifth load)
+        const int L = i * 8 + c.wave;
+        if (L < 24) {
+            c.run_src[i] = uniform(w_tile + (size_t) (L / 12) * (kCellsA * 16) + (size_t) (L % 12) * 1024);
+            c.run_step[i] = (size_t) 2 * kCellsA * 16;
+        } else {
+            c.run_src[i] = uniform(a_tile + (size_t) ((L - 24) / 6) * a_step + (size_t) ((L - 24) % 6) * 1024);
+            c.run_step[i] = 2 * a_step;
+        }
+    }
+    {
+        // fifth load: cells 2048 .. 2303 are the last 256 cells of the second group's activations, cells 2304 .. 2367
+        // the multipliers of the two groups
+        const int cell = kTailCell + c.wave * kTailLanes + (c.lane < kTailLanes ? c.lane : 0);
+        if (cell < kOffM) {
+            c.tail_src = a_tile + a_step + (size_t) (cell - (kOffB + kCellsB)) * 16;
+            c.tail_step = 2 * a_step;
+        } else {
+            const int gi = (cell - kOffM) / kCellsM, off = (cell - kOffM) % kCellsM;
+            c.tail_src = reinterpret_cast<const uint8_t *>(m4 + (size_t) gi * Mp + t0) + (size_t) off * 16;
+            c.tail_step = (size_t) 2 * Mp * sizeof(float);
+        }
+    }
+    const int panel = min(row_tile * 4 + c.wr, n_panels - 1);
+    c.k_src = kmul + (size_t) panel * ng * kPanelRows + 4 * (c.lane >> 5);
+
+    if (c.wave < 4) {
+        const int64_t n = (int64_t) row_tile * kTileRows + 64 * c.wave + c.lane;
+        load_to_lds_dword(s_w + (n < N ? n : N - 1), &s_pre[64 * c.wave]);
+    } else if (c.wave < 6) {
+        const int t = t0 + 64 * (c.wave - 4) + c.lane;
+        load_to_lds_dword(u + (t < M ? t : M - 1), &s_pre[kTileRows + 64 * (c.wave - 4)]);
+    }
+
+    float acc[2][2][16];
+    int32_t tot[2][2][16];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                acc[a][b][r] = kBias;
+                tot[a][b][r] = 0;
+            }
+        }
+    }
+    const bool hask = flags[0] & 1;
+    // fp32 rounding toward minus infinity for the folds (MODE bits 1:0); the MFMA sums are exact in any mode
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2" ::: "memory");
+    if (hask) {
+        body<true, GS>(c, s0, s1, s2, s3, acc, tot);
+    } else {
+        body<false, GS>(c, s0, s1, s2, s3, acc, tot);
+        flush(acc, tot);
+    }
+    // back to round to nearest even for the epilogue; the totals pass through the statement so that none of the
+    // conversions below can be scheduled in front of it
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0" ::: "memory");
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) asm volatile("" : "+v"(tot[a][b][r]));
+        }
+    }
+
+    // epilogue (reference patch line 176): y = ((float(total) * 16) * u) * s_w. Lane = one token (column of the MFMA
+    // result) and, per tile, rows 8 q + 4 (lane / 32) + 0 .. 3 for q = 0 .. 3.
+    const int h = c.lane >> 5;
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        const int tl = 64 * c.wc + 32 * b + (c.lane & 31);
+        const int t = t0 + tl;
+        if (t >= M) continue;
+        const float ut = s_pre[kTileRows + tl];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int rl = 64 * c.wr + 32 * a + 8 * q + 4 * h;
+                const int64_t n = (int64_t) row_tile * kTileRows + rl;
+                float *dst = y + (int64_t) t * ldy + n;
+                const float4 sw = *reinterpret_cast<const float4 *>(&s_pre[rl]);
+                const float swv[4] = { sw.x, sw.y, sw.z, sw.w };
+                float o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[i] = (((float) tot[a][b][4 * q + i] * 16.0f) * ut) * swv[i];
+                if (n + 3 < N && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
+                    typedef float v4f __attribute__((ext_vector_type(4)));
+                    __builtin_nontemporal_store(v4f{ o[0], o[1], o[2], o[3] }, reinterpret_cast<v4f *>(dst));
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        if (n + i < N) dst[i] = o[i];
+                    }
+                }
+            }
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_gemm6(const GemmArgs &a, hipStream_t stream) {
+    const uint8_t *p = a.prepared;
+    const int n_row_tiles = a.L.n_rtiles;
+    const int n_tok_tiles = a.Mp / kTileTok;
+    const int n_tiles = n_row_tiles * n_tok_tiles;
+    const int super_tiles = n_tok_tiles % 4 == 0 && n_row_tiles % 8 == 0;
+    const float *m4 = reinterpret_cast<const float *>(a.act8 + act6_plane_bytes(a.L.ng, a.Mp));
+#define RQ_LAUNCH6(GS)                                                                                              \
+    hipLaunchKernelGGL(rq_gemm6_kernel<GS>, dim3(n_tiles), dim3(kThreads), 0, stream, p + a.L.off_w6,                 \
+                       reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,                           \
+                       reinterpret_cast<const int32_t *>(p + a.L.off_flags), a.act8, m4, a.u, a.y, a.ldy, a.L.N, a.M, \
+                       a.Mp, a.L.ng, a.L.n_panels, n_tok_tiles, n_tiles, super_tiles)
+    if (a.groups_per_fold == 1) RQ_LAUNCH6(1);
+    else if (a.groups_per_fold == 2) RQ_LAUNCH6(2);
+    else RQ_LAUNCH6(4);
+#undef RQ_LAUNCH6
+    return hipGetLastError();
+}
+
+}  // namespace rq

@@ -237,6 +237,31 @@ rq_rotate_quant_kernel(const RotQuantArgs a) {
         const int z = (int) zf;
         const float *sp = buf + padi(8 * wc);
         const float f[8] = { sp[0], sp[1], sp[2], sp[3], sp[4], sp[5], sp[6], sp[7] };
+        if (a.mode == kActI8 && a.single == 2) {
+            // fp6 fragment plane: q - z as sign and magnitude, six bits each (as fp6 E2M3 the value is (q - z) / 8);
+            // this word's 48 bits are bytes 6 (w % 4) .. of the 24 bytes that lane token % 32 + 32 * (half of the group)
+            // holds in the fragment of 32 tokens: bytes 0 .. 15 at lane * 16, bytes 16 .. 23 at 1024 + lane * 8
+            uint64_t bits = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int d = (int) (fminf(fmaxf(rintf(f[j] * inv) + zf, 0.0f), 15.0f) - zf);
+                const uint32_t code = d < 0 ? (32u | (uint32_t) (-d)) : (uint32_t) d;
+                bits |= (uint64_t) code << (6 * j);
+            }
+            if (on) {
+                const int c8 = w & 7;
+                const int lane = (t & 31) + 32 * (c8 >> 2);
+                uint8_t *frag = reinterpret_cast<uint8_t *>(a.act) + ((size_t) g * (a.Mp >> 5) + (t >> 5)) * kFrag6;
+#pragma unroll
+                for (int i = 0; i < 3; ++i) {
+                    const int o = 6 * (c8 & 3) + 2 * i;   // byte of the lane's 24
+                    uint8_t *dst = o < 16 ? frag + lane * 16 + o : frag + 1024 + lane * 8 + (o - 16);
+                    *reinterpret_cast<uint16_t *>(dst) = (uint16_t) (bits >> (16 * i));
+                }
+                if (c8 == 0) a.m4[(size_t) g * a.Mp + t] = 4.0f * (float) mg;
+            }
+            continue;
+        }
         if (a.mode == kActI8 && a.single) {
             uint32_t even, odd;
             qz_of_word(f, inv, zf, even, odd);
