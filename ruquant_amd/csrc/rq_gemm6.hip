@@ -59,6 +59,7 @@ constexpr int kTailCell = 2048, kTailLanes = 40;
 static_assert(kTailCell + 8 * kTailLanes == kStageCells, "tail split");
 constexpr int kLoadsPerStep = 5;
 
+constexpr int kXposeStride = 68;               // floats between tokens of a wavefront's output block in LDS (64 rows + 4)
 constexpr float kBias = 12582912.0f;           // 1.5 x 2^23
 constexpr int kBiasBits = 0x4B400000;
 constexpr int kFlushSteps = 16;                // 32 groups
@@ -171,6 +172,12 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, int st, fl
     for (int gi = 0; gi < 2; ++gi) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
+#if RQ6_VARIANT == 3
+            for (int e = 0; e < 6; ++e) { A[gi][i][e] = c.lane * (e + gi + 1) + st; B[gi][i][e] = c.lane * (e + i + 3) + st; }
+            m4[gi][i] = 4.0f;
+            asm volatile("" : "+v"(A[gi][i]), "+v"(B[gi][i]));
+            continue;
+#endif
             A[gi][i] = fragment(s, kOffA + gi * kCellsA + (2 * c.wr + i) * (kFrag6 / 16), c.lane);
             B[gi][i] = fragment(s, kOffB + gi * kCellsB + (2 * c.wc + i) * (kFrag6 / 16), c.lane);
             m4[gi][i] = reinterpret_cast<const float *>(&s.cell[kOffM + gi * kCellsM])[64 * c.wc + 32 * i + (c.lane & 31)];
@@ -226,11 +233,14 @@ template <bool HASK, int GS>
 __device__ __forceinline__ void step(Ctx &c, const Stage &cur, Stage &refill, int st, float (&acc)[2][2][16],
                                      int32_t (&tot)[2][2][16], v16f (&carry)[2][2]) {
     // the loads of steps st + 1 and st + 2 may still be in flight
+#ifndef RQ6_VARIANT
+#define RQ6_VARIANT 0
+#endif
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerStep) : "memory");
-    __builtin_amdgcn_s_barrier();
+    if (RQ6_VARIANT != 4) __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    fetch(c, refill, st + 3);
-    compute<HASK, GS>(c, cur, st, acc, tot, carry);
+    if (RQ6_VARIANT != 1) fetch(c, refill, st + 3);
+    if (RQ6_VARIANT != 2) compute<HASK, GS>(c, cur, st, acc, tot, carry);
 }
 
 __device__ __forceinline__ void flush(float (&acc)[2][2][16], int32_t (&tot)[2][2][16]) {
@@ -273,10 +283,9 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
                 const int32_t *__restrict__ flags, const uint8_t *__restrict__ act6, const float *__restrict__ m4,
                 const float *__restrict__ u, float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng,
                 int n_panels, int n_tok_tiles, int n_tiles, int super_tiles) {
-    __shared__ Stage s0;
-    __shared__ Stage s1;
-    __shared__ Stage s2;
-    __shared__ Stage s3;
+    __shared__ Stage ring[kRing];
+    Stage &s0 = ring[0], &s1 = ring[1], &s2 = ring[2], &s3 = ring[3];
+    static_assert(8 * 64 * kXposeStride * 4 <= sizeof(ring), "the epilogue's output blocks fit the ring");
     // the epilogue's operands, fetched ahead of the first groups: the scales of the tile's 256 rows, then the units of
     // its 128 tokens
     __shared__ __align__(16) float s_pre[kTileRows + kTileTok];
@@ -301,15 +310,21 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
         }
     }
     const int tid = threadIdx.x;
+#ifdef RQ6_STAMPS
+    const long long ts0 = clock64();
+#endif
     Ctx c;
     c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     c.wr = c.wave & 3;
     c.wc = c.wave >> 2;
     c.lane = tid & 63;
     c.n_steps = ng / 2;
-    const uint8_t *w_tile = w6 + (size_t) row_tile * ng * (kCellsA * 16);   // this tile's rows, group 0
+#ifndef RQ6_SRC
+#define RQ6_SRC 0
+#endif
+    const uint8_t *w_tile = w6 + (size_t) ((RQ6_SRC & 1) ? 0 : row_tile) * ng * (kCellsA * 16);   // this tile's rows, group 0
     const size_t a_step = (size_t) (Mp / 32) * kFrag6;                       // bytes between groups of the activation plane
-    const uint8_t *a_tile = act6 + (size_t) (t0 / 32) * kFrag6;              // this tile's tokens, group 0
+    const uint8_t *a_tile = act6 + (size_t) (((RQ6_SRC & 2) ? 0 : t0) / 32) * kFrag6;              // this tile's tokens, group 0
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         // run L of the stage: runs 0 .. 23 are the weights of the step's two groups (12 each), 24 .. 35 the activations
@@ -361,6 +376,9 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
         }
     }
     const bool hask = flags[0] & 1;
+#ifdef RQ6_STAMPS
+    const long long ts1 = clock64();
+#endif
     // fp32 rounding toward minus infinity for the folds (MODE bits 1:0); the MFMA sums are exact in any mode
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2" ::: "memory");
     if (hask) {
@@ -369,6 +387,9 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
         body<false, GS>(c, s0, s1, s2, s3, acc, tot);
         flush(acc, tot);
     }
+#ifdef RQ6_STAMPS
+    const long long ts2 = clock64();
+#endif
     // back to round to nearest even for the epilogue; the totals pass through the statement so that none of the
     // conversions below can be scheduled in front of it
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0" ::: "memory");
@@ -381,39 +402,62 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
         }
     }
 
-    // epilogue (reference patch line 176): y = ((float(total) * 16) * u) * s_w. Lane = one token (column of the MFMA
-    // result) and, per tile, rows 8 q + 4 (lane / 32) + 0 .. 3 for q = 0 .. 3.
+    // epilogue (reference patch line 176): y = ((float(total) * 16) * u) * s_w. In the MFMA result a lane holds one
+    // token (column) and, per tile, rows 8 q + 4 (lane / 32) + 0 .. 3 for q = 0 .. 3: stored as they are, a wavefront's
+    // stores would be 32-byte pieces of 32 different rows of y (a third of the kernel's time went there). So every
+    // wavefront turns its 64 x 64 outputs through LDS (the ring is free now) and writes 256 contiguous bytes per token.
+    __syncthreads();   // every wavefront is done reading the ring
+    float *xp = reinterpret_cast<float *>(&s0.cell[0]) + c.wave * (64 * kXposeStride);   // s0 .. s3 are one 148 KiB block
     const int h = c.lane >> 5;
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-        const int tl = 64 * c.wc + 32 * b + (c.lane & 31);
-        const int t = t0 + tl;
-        if (t >= M) continue;
-        const float ut = s_pre[kTileRows + tl];
+        const int tw = 32 * b + (c.lane & 31);   // token within the wavefront's 64
+        const float ut = s_pre[kTileRows + 64 * c.wc + tw];
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int rl = 64 * c.wr + 32 * a + 8 * q + 4 * h;
-                const int64_t n = (int64_t) row_tile * kTileRows + rl;
-                float *dst = y + (int64_t) t * ldy + n;
-                const float4 sw = *reinterpret_cast<const float4 *>(&s_pre[rl]);
-                const float swv[4] = { sw.x, sw.y, sw.z, sw.w };
-                float o[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) o[i] = (((float) tot[a][b][4 * q + i] * 16.0f) * ut) * swv[i];
-                if (n + 3 < N && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
-                    typedef float v4f __attribute__((ext_vector_type(4)));
-                    __builtin_nontemporal_store(v4f{ o[0], o[1], o[2], o[3] }, reinterpret_cast<v4f *>(dst));
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        if (n + i < N) dst[i] = o[i];
-                    }
-                }
+                const int rw = 32 * a + 8 * q + 4 * h;   // row within the wavefront's 64
+                const float4 sw = *reinterpret_cast<const float4 *>(&s_pre[64 * c.wr + rw]);
+                float4 o;
+                o.x = (((float) tot[a][b][4 * q + 0] * 16.0f) * ut) * sw.x;
+                o.y = (((float) tot[a][b][4 * q + 1] * 16.0f) * ut) * sw.y;
+                o.z = (((float) tot[a][b][4 * q + 2] * 16.0f) * ut) * sw.z;
+                o.w = (((float) tot[a][b][4 * q + 3] * 16.0f) * ut) * sw.w;
+                *reinterpret_cast<float4 *>(&xp[tw * kXposeStride + rw]) = o;
             }
         }
     }
+    // (a wavefront reads back only what it wrote itself: its LDS operations complete in order)
+    const int64_t n = (int64_t) row_tile * kTileRows + 64 * c.wr + 4 * (c.lane & 15);
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+        const int tw = 4 * it + (c.lane >> 4);
+        const int t = t0 + 64 * c.wc + tw;
+        const float4 o = *reinterpret_cast<const float4 *>(&xp[tw * kXposeStride + 4 * (c.lane & 15)]);
+        if (t >= M) continue;
+        float *dst = y + (int64_t) t * ldy + n;
+        if (n + 3 < N && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
+            // the output is written once and not read back by this launch: non-temporal
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            __builtin_nontemporal_store(v4f{ o.x, o.y, o.z, o.w }, reinterpret_cast<v4f *>(dst));
+        } else {
+            const float ov[4] = { o.x, o.y, o.z, o.w };
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (n + i < N) dst[i] = ov[i];
+            }
+        }
+    }
+#ifdef RQ6_STAMPS
+    __syncthreads();
+    if (tid == 0) {
+        long long *dbg = reinterpret_cast<long long *>(y) + (size_t) blockIdx.x * 8;
+        unsigned hwid = __builtin_amdgcn_s_getreg((32 - 1) << 11 | 0 << 6 | 4);
+        unsigned xcc = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 0 << 6 | 20);
+        dbg[0] = ts0; dbg[1] = ts1; dbg[2] = ts2; dbg[3] = clock64(); dbg[4] = hwid; dbg[5] = xcc; dbg[6] = row_tile; dbg[7] = t0;
+    }
+#endif
 }
 
 }  // namespace
