@@ -253,6 +253,10 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     } else if (path == kPathSkinny) {
         q.zero_ptr = reinterpret_cast<int32_t *>(wsb + W.off_tot);
         q.zero_ints = 2 * M * (int64_t) ((Ncells + kPanelRows - 1) / kPanelRows * kPanelRows);
+    } else if (fp6) {
+        // the arrival counters of the tiles the fp6 GEMM cuts along K
+        q.zero_ptr = reinterpret_cast<int32_t *>(wsb + W.off_tot);
+        q.zero_ints = (int64_t) (kGemm6CounterBytes / sizeof(int32_t));
     }
     hipError_t e = hipSuccess;
     if (stages & 1) {
@@ -303,6 +307,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             g.M = (int) M;
             g.Mp = (int) W.Mp;
             g.groups_per_fold = G / kGroup;
+            g.cells = wsb + W.off_tot;
             e = fp6 ? launch_gemm6(g, stream) : launch_gemm(g, stream);
             if (e != hipSuccess) return (int) e;
         } else {

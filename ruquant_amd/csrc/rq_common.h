@@ -103,8 +103,10 @@ struct WorkspaceLayout {
     int64_t Mp;       // tokens padded to the GEMM tile
     int     chunks;   // ceil(M / 8)
     size_t  off_u, off_act, off_lohi, off_rpart, off_i8, off_tot, bytes;
-    size_t  tot_ints;
+    size_t  tot_ints;   // ints of the split-K cells at off_tot (two per cell)
 };
+
+size_t gemm6_cell_bytes_max(int64_t N, int64_t M, int ng);
 
 inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
     WorkspaceLayout W;
@@ -128,6 +130,12 @@ inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
     W.off_i8 = small ? off + gemv_form : off;
     off = align_up(off + (small ? gemv_form + act_i8 : act_i8), 256);
     W.tot_ints = (size_t) 2 * (M <= kGemvTokens ? kGemvTokens : kSkinnyTokens) * n_panels * kPanelRows;
+    if (M > kSkinnyTokens && gemm_fp6_enabled()) {
+        // the fp6 GEMM's arrival cells (the tiles it cuts along K); sized for the widest activation group's plan, which
+        // cuts the most
+        const size_t cb = gemm6_cell_bytes_max(N, M, ng);
+        if (cb / sizeof(int32_t) > W.tot_ints) W.tot_ints = cb / sizeof(int32_t);
+    }
     W.off_tot = off;
     off = align_up(off + W.tot_ints * sizeof(int32_t), 256);
     W.bytes = off;
@@ -251,10 +259,21 @@ struct GemmArgs {
     int64_t         ldy;
     int             M, Mp;
     int             groups_per_fold;   // 1; 2 or 4 when the activation groups are 128 or 256 wide
+    void           *cells;             // fp6 form: arrival counters (zero on entry, left zero) and slabs of the tiles cut along K
 };
 hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
 // the fp6 form: act8 = the fp6 fragment plane with the multipliers behind it; the weight needs the fp6 plane
 hipError_t launch_gemm6(const GemmArgs &a, hipStream_t stream);
+// How a launch of the fp6 form is cut: n_whole tiles (256 rows x 128 tokens) run whole, the rest in `parts` slices of
+// K each, which meet in cell_bytes of workspace: kGemm6CounterBytes of arrival counters (one int per cut tile: zero on
+// entry, left zero), then one slab of partial totals per slice (needs no clearing).
+constexpr int kPlanUnits = 256;
+constexpr size_t kGemm6CounterBytes = kPlanUnits * sizeof(int32_t);
+struct Gemm6Plan {
+    int    n_tiles, n_whole, parts;
+    size_t cell_bytes;
+};
+Gemm6Plan gemm6_plan(int64_t N, int64_t M, int ng, int groups_per_fold);
 
 // up to 64 tokens: MFMA arithmetic on a GEMV-shaped weight stream; same operands as the GEMM plus the split-K cells
 struct SkinnyArgs {

@@ -57,7 +57,11 @@ static_assert(kStageCells == 2368, "stage size");
 // cells) and 40 lanes' worth of a fifth (cells 2048 .. 2367: the rest of the activations and the multipliers).
 constexpr int kTailCell = 2048, kTailLanes = 40;
 static_assert(kTailCell + 8 * kTailLanes == kStageCells, "tail split");
+#ifndef RQ6_NOTAIL
 constexpr int kLoadsPerStep = 5;
+#else
+constexpr int kLoadsPerStep = 4;
+#endif
 
 constexpr int kXposeStride = 68;               // floats between tokens of a wavefront's output block in LDS (64 rows + 4)
 constexpr float kBias = 12582912.0f;           // 1.5 x 2^23
@@ -115,7 +119,8 @@ struct Ctx {
     size_t tail_step;        // its advance per step
     const uint8_t *k_src;    // weight multipliers of this wavefront's panel, row offset of the lane's first quad
     int wave, wr, wc, lane;
-    int n_steps;
+    int n_steps;             // steps (two groups each) of this workgroup
+    int g0;                  // its first group
 };
 
 // fetch of the next step (two groups) into stage s, then advance the sources; past the last step they stay where they
@@ -128,7 +133,9 @@ __device__ __forceinline__ void fetch(Ctx &c, Stage &s, int st) {
         load_run(c.run_src[i], lane_off, &s.cell[(i * 8 + c.wave) * 64]);
         c.run_src[i] = uniform(c.run_src[i] + (more ? c.run_step[i] : 0));
     }
+#ifndef RQ6_NOTAIL
     load_cells(c.tail_src, &s.cell[kTailCell + c.wave * kTailLanes], ((uint64_t) 1 << kTailLanes) - 1);
+#endif
     c.tail_src += more ? c.tail_step : 0;
 }
 
@@ -172,7 +179,7 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, int st, fl
     for (int gi = 0; gi < 2; ++gi) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-#if RQ6_VARIANT == 3
+#if RQ6_VARIANT == 3 || RQ6_VARIANT == 5
             for (int e = 0; e < 6; ++e) { A[gi][i][e] = c.lane * (e + gi + 1) + st; B[gi][i][e] = c.lane * (e + i + 3) + st; }
             m4[gi][i] = 4.0f;
             asm volatile("" : "+v"(A[gi][i]), "+v"(B[gi][i]));
@@ -207,7 +214,7 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, int st, fl
                 fold_fast(P, m4[prev_gi][prev_b], acc[prev_a][prev_b]);
             } else {
                 // the multiplier of the group's first run (reference patch line 171: RQ_W_MULT_G(sum, sg << (2 - lsub)))
-                const int g = (GS == 4 ? 2 * (st & ~1) : 2 * st) + prev_gi;
+                const int g = c.g0 + (GS == 4 ? 2 * (st & ~1) : 2 * st) + prev_gi;
                 int k16[16];
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
@@ -223,8 +230,12 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, int st, fl
             prev_a = (un >> 1) & 1;
             prev_b = un & 1;
         }
-        // a unit's MFMAs and the previous unit's fold stay together: left alone, the scheduler issues all the
-        // (independent) MFMAs of a step first, and their results (16 registers each) spill
+        // A unit's MFMAs and the previous unit's fold stay together, MFMAs first: the fold then runs while the matrix
+        // pipe works on the next unit. (Left alone, the scheduler issues all the independent MFMAs of a step first and
+        // their results, 16 registers each, spill; with a plain barrier it puts the fold in front of the MFMA, so that
+        // every fold waits for the MFMA issued right before it.)
+        if (un < kUnits) __builtin_amdgcn_sched_group_barrier(0x008, kRuns, 0);   // MFMA
+        if (un > 0 && folds && !HASK) __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);   // VALU
         __builtin_amdgcn_sched_barrier(0);
     }
 }
@@ -237,9 +248,9 @@ __device__ __forceinline__ void step(Ctx &c, const Stage &cur, Stage &refill, in
 #define RQ6_VARIANT 0
 #endif
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerStep) : "memory");
-    if (RQ6_VARIANT != 4) __builtin_amdgcn_s_barrier();
+    if (RQ6_VARIANT != 4 && RQ6_VARIANT != 5 && RQ6_VARIANT != 6) __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (RQ6_VARIANT != 1) fetch(c, refill, st + 3);
+    if (RQ6_VARIANT != 1 && RQ6_VARIANT != 5 && RQ6_VARIANT != 7) fetch(c, refill, st + 3);
     if (RQ6_VARIANT != 2) compute<HASK, GS>(c, cur, st, acc, tot, carry);
 }
 
@@ -277,27 +288,145 @@ __device__ __forceinline__ void body(Ctx &c, Stage &s0, Stage &s1, Stage &s2, St
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the refetches of the last steps
 }
 
+// ---- groups of 64 (the common case): the same steps with the LDS reads taken out of the critical path.
+// The operands of a group are read from LDS while the previous group is being computed: the reads of a step's second
+// group are issued in front of the first group's MFMAs, and the wait for the next stage (vmcnt + barrier) sits between
+// the two groups, so that the next step's first group can be read behind the second group's MFMAs. (With all reads at
+// the top of a step every wavefront waited for 12 KiB from LDS at the same moment, right behind the barrier: a
+// quarter of the step.)
+struct Operands {
+    v8i A[2], B[2];
+    float m4[2];
+};
+
+__device__ __forceinline__ void read_operands(const Ctx &c, const Stage &s, int gi, Operands &o) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        o.A[i] = fragment(s, kOffA + gi * kCellsA + (2 * c.wr + i) * (kFrag6 / 16), c.lane);
+        o.B[i] = fragment(s, kOffB + gi * kCellsB + (2 * c.wc + i) * (kFrag6 / 16), c.lane);
+        o.m4[i] = reinterpret_cast<const float *>(&s.cell[kOffM + gi * kCellsM])[64 * c.wc + 32 * i + (c.lane & 31)];
+    }
+}
+
+// the four tiles of one group; the fold of a tile runs behind the MFMA of the next one, the last tile's result is
+// handed to the next group (P, pm, and the tile it belongs to is always (1, 1))
+template <bool HASK>
+__device__ __forceinline__ void group_units(const Ctx &c, const Operands &o, int g, v16f &P, float &pm,
+                                            float (&acc)[2][2][16], int32_t (&tot)[2][2][16]) {
+    const v16f zero = {};
+#pragma unroll
+    for (int un = 0; un < 4; ++un) {
+        const int a = un >> 1, b = un & 1;
+        const int pa = un == 0 ? 1 : (un - 1) >> 1, pb = un == 0 ? 1 : (un - 1) & 1;
+        const v16f S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.A[a], o.B[b], zero, 2, 2, 0, 0, 0, 0);
+        if (!HASK) {
+            fold_fast(P, pm, acc[pa][pb]);
+        } else {
+            const int pg = un == 0 ? g - 1 : g;   // (a workgroup's first fold adds nothing: P and pm start as zero)
+            int k16[16];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t k4 = *reinterpret_cast<const uint32_t *>(c.k_src + (size_t) (pg < 0 ? 0 : pg) * kPanelRows + 32 * pa + 8 * q);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) k16[4 * q + i] = (k4 >> (8 * i)) & 0xFF;
+            }
+            fold_k(P, pm, k16, tot[pa][pb]);
+        }
+        P = S;
+        pm = o.m4[b];
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                // MFMA
+        if (!HASK) __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);    // VALU: the fold
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+template <bool HASK>
+__device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, Stage &s3, float (&acc)[2][2][16],
+                                       int32_t (&tot)[2][2][16]) {
+    Stage *ring[kRing] = { &s0, &s1, &s2, &s3 };
+    Operands X, Y;
+    v16f P = {};
+    float pm = 0.0f;
+    fetch(c, s0, 0);
+    fetch(c, s1, 1);
+    fetch(c, s2, 2);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerStep) : "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    read_operands(c, s0, 0, X);
+    for (int st0 = 0; st0 < c.n_steps; st0 += kRing) {
+#pragma unroll
+        for (int j = 0; j < kRing; ++j) {
+            const int st = st0 + j;
+            if (j > 0 && st >= c.n_steps) break;   // (wave-uniform)
+            const Stage &cur = *ring[j];
+            const Stage &next = *ring[(j + 1) % kRing];
+            Stage &refill = *ring[(j + 3) % kRing];
+            read_operands(c, cur, 1, Y);
+            __builtin_amdgcn_sched_barrier(0);
+            group_units<HASK>(c, X, c.g0 + 2 * st, P, pm, acc, tot);
+            // stage st + 1 is whole once every wavefront has seen its own loads of it arrive (those of step st + 2
+            // may still be in flight); stage st - 1 is then free for step st + 3
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerStep) : "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            fetch(c, refill, st + 3);
+            read_operands(c, next, 0, X);   // (past the last step: stale cells, never used)
+            __builtin_amdgcn_sched_barrier(0);
+            group_units<HASK>(c, Y, c.g0 + 2 * st + 1, P, pm, acc, tot);
+        }
+        if (!HASK && ((st0 / kRing + 1) % (kFlushSteps / kRing)) == 0) flush(acc, tot);
+    }
+    // the last tile of the last group
+    if (!HASK) {
+        fold_fast(P, pm, acc[1][1]);
+    } else {
+        int k16[16];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t k4 = *reinterpret_cast<const uint32_t *>(c.k_src + (size_t) (c.g0 + 2 * c.n_steps - 1) * kPanelRows + 32 + 8 * q);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) k16[4 * q + i] = (k4 >> (8 * i)) & 0xFF;
+        }
+        fold_k(P, pm, k16, tot[1][1]);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the refetches of the last steps
+}
+
 template <int GS>
 __global__ void __launch_bounds__(kThreads)
 rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                 const int32_t *__restrict__ flags, const uint8_t *__restrict__ act6, const float *__restrict__ m4,
                 const float *__restrict__ u, float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng,
-                int n_panels, int n_tok_tiles, int n_tiles, int super_tiles) {
+                int n_panels, int n_tok_tiles, int n_tiles, int super_tiles, int n_whole, int parts,
+                int *__restrict__ counters, unsigned long long *__restrict__ slabs) {
     __shared__ Stage ring[kRing];
     Stage &s0 = ring[0], &s1 = ring[1], &s2 = ring[2], &s3 = ring[3];
     static_assert(8 * 64 * kXposeStride * 4 <= sizeof(ring), "the epilogue's output blocks fit the ring");
     // the epilogue's operands, fetched ahead of the first groups: the scales of the tile's 256 rows, then the units of
     // its 128 tokens
-    __shared__ __align__(16) float s_pre[kTileRows + kTileTok];
+    __shared__ __align__(16) float s_pre[kTileRows + kTileTok + 4];   // (+ a word for the arrival count of a slice)
 
     // Workgroups go to the eight XCDs round robin: every XCD gets a contiguous run of tiles, visited in super-tiles of
     // 8 row tiles x 4 token tiles (the 32 workgroups an XCD runs at a time then share 8 weight tiles and 4 activation
     // tiles in its L2), or with the token tiles running fastest where the launch is not made of whole super-tiles.
-    int row_tile, t0;
+    // The first n_whole workgroups take a whole tile each. The tiles after them (fewer than would fill the chip once)
+    // are cut along K into `parts` slices each, one workgroup per slice, which meet through memory (see the epilogue).
+    int row_tile, t0, part = 0, slot = 0;
     {
         int v = blockIdx.x;
-        const int per_xcd = n_tiles / kXcds;
-        if (v < per_xcd * kXcds) v = (v % kXcds) * per_xcd + v / kXcds;
+        if (v < n_whole) {
+            const int per_xcd = n_whole / kXcds;
+            if (v < per_xcd * kXcds) v = (v % kXcds) * per_xcd + v / kXcds;
+        } else {
+            // slices: an XCD gets a contiguous run of (tile, part) pairs, parts running slowest within the run, so that
+            // neighbouring tiles' slices of the same stretch of K are resident together
+            int j = v - n_whole;
+            const int n_sl = (n_tiles - n_whole) * parts, per_xcd = n_sl / kXcds;
+            if (j < per_xcd * kXcds) j = (j % kXcds) * per_xcd + j / kXcds;
+            v = n_whole + j / parts;
+            part = j - (j / parts) * parts;
+        }
         if (super_tiles) {
             const int s = v >> 5, i = v & 31;
             const int spr = n_tok_tiles >> 2;
@@ -308,7 +437,12 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
             row_tile = v / n_tok_tiles;
             t0 = (v - row_tile * n_tok_tiles) * kTileTok;
         }
+        slot = v - n_whole;
     }
+    const bool sliced = (int) blockIdx.x >= n_whole;
+    // this workgroup's steps (two groups each) of the tile's ng / 2
+    const int s_begin = sliced ? (int) ((int64_t) (ng / 2) * part / parts) : 0;
+    const int s_end = sliced ? (int) ((int64_t) (ng / 2) * (part + 1) / parts) : ng / 2;
     const int tid = threadIdx.x;
 #ifdef RQ6_STAMPS
     const long long ts0 = clock64();
@@ -318,12 +452,17 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
     c.wr = c.wave & 3;
     c.wc = c.wave >> 2;
     c.lane = tid & 63;
-    c.n_steps = ng / 2;
+    c.n_steps = s_end - s_begin;
+    c.g0 = 2 * s_begin;
 #ifndef RQ6_SRC
 #define RQ6_SRC 0
 #endif
     const uint8_t *w_tile = w6 + (size_t) ((RQ6_SRC & 1) ? 0 : row_tile) * ng * (kCellsA * 16);   // this tile's rows, group 0
+#ifndef RQ6_BCONTIG
     const size_t a_step = (size_t) (Mp / 32) * kFrag6;                       // bytes between groups of the activation plane
+#else
+    const size_t a_step = (size_t) 4 * kFrag6;
+#endif
     const uint8_t *a_tile = act6 + (size_t) (((RQ6_SRC & 2) ? 0 : t0) / 32) * kFrag6;              // this tile's tokens, group 0
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -331,11 +470,11 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
         // (6 each; the last four belong to the fifth load)
         const int L = i * 8 + c.wave;
         if (L < 24) {
-            c.run_src[i] = uniform(w_tile + (size_t) (L / 12) * (kCellsA * 16) + (size_t) (L % 12) * 1024);
             c.run_step[i] = (size_t) 2 * kCellsA * 16;
+            c.run_src[i] = uniform(w_tile + (size_t) (L / 12) * (kCellsA * 16) + (size_t) (L % 12) * 1024 + s_begin * c.run_step[i]);
         } else {
-            c.run_src[i] = uniform(a_tile + (size_t) ((L - 24) / 6) * a_step + (size_t) ((L - 24) % 6) * 1024);
             c.run_step[i] = 2 * a_step;
+            c.run_src[i] = uniform(a_tile + (size_t) ((L - 24) / 6) * a_step + (size_t) ((L - 24) % 6) * 1024 + s_begin * c.run_step[i]);
         }
     }
     {
@@ -343,12 +482,12 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
         // the multipliers of the two groups
         const int cell = kTailCell + c.wave * kTailLanes + (c.lane < kTailLanes ? c.lane : 0);
         if (cell < kOffM) {
-            c.tail_src = a_tile + a_step + (size_t) (cell - (kOffB + kCellsB)) * 16;
             c.tail_step = 2 * a_step;
+            c.tail_src = a_tile + a_step + (size_t) (cell - (kOffB + kCellsB)) * 16 + s_begin * c.tail_step;
         } else {
             const int gi = (cell - kOffM) / kCellsM, off = (cell - kOffM) % kCellsM;
-            c.tail_src = reinterpret_cast<const uint8_t *>(m4 + (size_t) gi * Mp + t0) + (size_t) off * 16;
             c.tail_step = (size_t) 2 * Mp * sizeof(float);
+            c.tail_src = reinterpret_cast<const uint8_t *>(m4 + (size_t) gi * Mp + t0) + (size_t) off * 16 + s_begin * c.tail_step;
         }
     }
     const int panel = min(row_tile * 4 + c.wr, n_panels - 1);
@@ -382,9 +521,11 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
     // fp32 rounding toward minus infinity for the folds (MODE bits 1:0); the MFMA sums are exact in any mode
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2" ::: "memory");
     if (hask) {
-        body<true, GS>(c, s0, s1, s2, s3, acc, tot);
+        if constexpr (GS == 1) body64<true>(c, s0, s1, s2, s3, acc, tot);
+        else body<true, GS>(c, s0, s1, s2, s3, acc, tot);
     } else {
-        body<false, GS>(c, s0, s1, s2, s3, acc, tot);
+        if constexpr (GS == 1) body64<false>(c, s0, s1, s2, s3, acc, tot);
+        else body<false, GS>(c, s0, s1, s2, s3, acc, tot);
         flush(acc, tot);
     }
 #ifdef RQ6_STAMPS
@@ -399,6 +540,42 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
         for (int b = 0; b < 2; ++b) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) asm volatile("" : "+v"(tot[a][b][r]));
+        }
+    }
+
+    if (sliced) {
+        // A slice of K: its totals go to a slab of their own (64 ints per thread, written through to memory at
+        // device scope: the slices of a tile run on different XCDs, each with its own L2), then one atomic per
+        // workgroup counts the arrival. The workgroup that completes the count adds the other slices' slabs to the
+        // totals it still holds and goes on to the epilogue; the others are done. (An atomic per output instead,
+        // accumulating in 64-bit arrival cells, cost more than the slicing gained: 8 M device-scope atomics.)
+        unsigned long long *slab = slabs + ((size_t) slot * parts + part) * (kTileRows * kTileTok / 2);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const int a = i >> 4, b = (i >> 3) & 1, r = 2 * (i & 7);
+            const unsigned long long two = (unsigned long long) (uint32_t) tot[a][b][r] | (unsigned long long) (uint32_t) tot[a][b][r + 1] << 32;
+            __hip_atomic_store(slab + (size_t) i * kThreads + tid, two, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's stores have reached memory
+        __syncthreads();                                    // ... and everybody else's
+        int *s_flag = reinterpret_cast<int *>(&s_pre[kTileRows + kTileTok]);
+        if (tid == 0) {
+            const int before = __hip_atomic_fetch_add(counters + slot, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (before == parts - 1) __hip_atomic_store(counters + slot, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *s_flag = before;
+        }
+        __syncthreads();
+        if (*s_flag != parts - 1) return;
+        for (int pp = 0; pp < parts; ++pp) {
+            if (pp == part) continue;
+            const unsigned long long *other = slabs + ((size_t) slot * parts + pp) * (kTileRows * kTileTok / 2);
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                const int a = i >> 4, b = (i >> 3) & 1, r = 2 * (i & 7);
+                const unsigned long long two = __hip_atomic_load(other + (size_t) i * kThreads + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                tot[a][b][r] += (int32_t) (uint32_t) two;
+                tot[a][b][r + 1] += (int32_t) (uint32_t) (two >> 32);
+            }
         }
     }
 
@@ -462,18 +639,61 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
 
 }  // namespace
 
+Gemm6Plan gemm6_plan(int64_t N, int64_t M, int ng, int groups_per_fold) {
+    Gemm6Plan pl;
+    const int n_row_tiles = (int) ((N + kTileRows - 1) / kTileRows);
+    const int n_tok_tiles = (int) ((M + kTileTok - 1) / kTileTok);
+    pl.n_tiles = n_row_tiles * n_tok_tiles;
+    pl.n_whole = pl.n_tiles;
+    pl.parts = 1;
+    // Whole rounds of the chip run a tile per workgroup. What is left over (fewer tiles than compute units) would
+    // keep the chip busy for one more whole tile time; cut along K into `parts` slices per tile it takes 1 / parts of
+    // that. (The count of compute units is taken as the 256 of the part this library is written for: the plan must
+    // not depend on the device, because the workspace is sized from it.)
+    const int left = pl.n_tiles % kPlanUnits;
+    if (left > 0 && kPlanUnits / left >= 2) {
+        int parts = kPlanUnits / left;
+        const int steps = ng / 2;
+        if (parts > steps / 2) parts = steps / 2;               // at least two steps per slice
+        // wider activation groups: a slice holds whole groups and an even number of steps
+        if (groups_per_fold > 1) {
+            while (parts > 1 && steps % (2 * parts) != 0) --parts;
+        }
+        if (parts >= 2) {
+            pl.parts = parts;
+            pl.n_whole = pl.n_tiles - left;
+        }
+    }
+    // one arrival counter per cut tile, then a slab of 256 x 128 ints per slice
+    pl.cell_bytes = pl.parts > 1 ? kGemm6CounterBytes + (size_t) (pl.n_tiles - pl.n_whole) * pl.parts * kTileRows * kTileTok * sizeof(int32_t) : 0;
+    return pl;
+}
+
+size_t gemm6_cell_bytes_max(int64_t N, int64_t M, int ng) {
+    size_t best = 0;
+    for (int gf = 1; gf <= 4; gf *= 2) {
+        const size_t b = gemm6_plan(N, M, ng, gf).cell_bytes;
+        if (b > best) best = b;
+    }
+    return best;
+}
+
 hipError_t launch_gemm6(const GemmArgs &a, hipStream_t stream) {
     const uint8_t *p = a.prepared;
     const int n_row_tiles = a.L.n_rtiles;
     const int n_tok_tiles = a.Mp / kTileTok;
-    const int n_tiles = n_row_tiles * n_tok_tiles;
+    const Gemm6Plan pl = gemm6_plan(a.L.N, a.M, a.L.ng, a.groups_per_fold);
+    if (pl.n_tiles != n_row_tiles * n_tok_tiles || (pl.parts > 1 && a.cells == nullptr)) return hipErrorInvalidValue;
     const int super_tiles = n_tok_tiles % 4 == 0 && n_row_tiles % 8 == 0;
+    const int grid = pl.n_whole + (pl.n_tiles - pl.n_whole) * pl.parts;
     const float *m4 = reinterpret_cast<const float *>(a.act8 + act6_plane_bytes(a.L.ng, a.Mp));
 #define RQ_LAUNCH6(GS)                                                                                              \
-    hipLaunchKernelGGL(rq_gemm6_kernel<GS>, dim3(n_tiles), dim3(kThreads), 0, stream, p + a.L.off_w6,                 \
+    hipLaunchKernelGGL(rq_gemm6_kernel<GS>, dim3(grid), dim3(kThreads), 0, stream, p + a.L.off_w6,                    \
                        reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,                           \
                        reinterpret_cast<const int32_t *>(p + a.L.off_flags), a.act8, m4, a.u, a.y, a.ldy, a.L.N, a.M, \
-                       a.Mp, a.L.ng, a.L.n_panels, n_tok_tiles, n_tiles, super_tiles)
+                       a.Mp, a.L.ng, a.L.n_panels, n_tok_tiles, pl.n_tiles, super_tiles, pl.n_whole, pl.parts,      \
+                       reinterpret_cast<int *>(a.cells),                                                             \
+                       reinterpret_cast<unsigned long long *>(reinterpret_cast<uint8_t *>(a.cells) + kGemm6CounterBytes))
     if (a.groups_per_fold == 1) RQ_LAUNCH6(1);
     else if (a.groups_per_fold == 2) RQ_LAUNCH6(2);
     else RQ_LAUNCH6(4);
