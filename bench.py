@@ -12,14 +12,17 @@ Prints one JSON line. Besides the contract fields it carries
                    stream), against the HBM peak,
   roofline_m2048 : the tiled MFMA GEMM alone at M = 2048 (K = 5120, N = 17408), against the dense int8 MFMA peak: the
                    second half of the metric,
-  cpu_baseline   : the CPU oracle (a bit-identical restatement of the ggml-cpu reference path) on the host cores,
+  cpu_baseline   : the CPU oracle (a bit-identical restatement of the ggml-cpu reference path) on the host cores, on
+                   the headline problem,
+  cpu_baseline_m2048 : one whole pass of the same oracle over the M = 2048 problem (its result is also what the GPU's
+                   output of that problem is compared with, bit for bit),
   extra          : the same measurements for the other benchmark shapes (the N = 5120 decode shapes, the K = 17408 down
                    projection, the reference's perf-mode shape 6144 x 5120), the seven matmuls of one transformer
                    layer at 16 tokens and at one token, run in the layer's dataflow, and `peaks`: what this machine
                    delivers to plain probe kernels in the same run (a streaming read of the headline's byte count, a
-                   pure v_mfma_i32_16x16x64_i8 loop, vector-ALU instructions beside MFMAs in one wavefront and in two
-                   wavefronts that share a SIMD, an empty launch).
-Every time is the median over batches of back-to-back launches captured in one HIP graph.
+                   pure MFMA loop of every form the kernels use or were weighed against, vector-ALU instructions
+                   beside MFMAs in one wavefront and in two wavefronts that share a SIMD, an empty launch).
+Every time is the median over 11 batches of back-to-back launches captured in one HIP graph.
 """
 import argparse
 import json
@@ -59,19 +62,21 @@ def algorithmic_bytes(K, N, M):
 class Problem:
     """One (K, N, M) W4A4H problem with rotating weight copies and a preallocated workspace."""
 
-    def __init__(self, K, N, M, act_kind, clip, seed, min_rotate_bytes=320 << 20, dev="cuda:0"):
+    def __init__(self, K, N, M, act_kind, clip, seed, min_rotate_bytes=320 << 20, dev="cuda:0", type_=None):
         import numpy as np
         import torch
         import ruquant_amd as rq
         from ruquant_amd import synth
         self.K, self.N, self.M = K, N, M
         self.rq, self.torch = rq, torch
-        self.type = rq.TYPE_W4A4H
+        self.type = rq.TYPE_W4A4H if type_ is None else type_
         self.blocks = synth.random_weight_blocks(N, K, seed, self.type, clip=clip if clip != 1.0 else 0.0)
         self.x_host = synth.activations(act_kind, M, K, seed)
         self.weight = rq.W4A4Weight(self.blocks, self.type, dev, keep_blocks=False)
         self.clip = float(np.float32(clip))
-        n_copies = max(1, -(-min_rotate_bytes // (N * K // 2)))
+        # bytes of a prepared weight that one call reads: the int4 codes, or the fp6 plane of the wide-batch kernel
+        fp6 = M > 64 and os.environ.get("RQ_GEMM_FP6", "1") != "0"
+        n_copies = max(1, -(-min_rotate_bytes // (N * K * 3 // 4 if fp6 else N * K // 2)))
         self.prepared = [self.weight.prepared] + [self.weight.prepared.clone() for _ in range(n_copies - 1)]
         self.x = torch.from_numpy(self.x_host).to(dev)
         self.y = torch.empty((M, N), dtype=torch.float32, device=dev)
@@ -137,15 +142,20 @@ class Problem:
         wall_ms = (time.perf_counter() - t0) * 1e3 / steps
         return gpu_ms, wall_ms
 
-    def median_timed(self, steps, warmup, stages, batches=7):
+    def stage_mask(self):
+        """which stages launch kernels for this problem (a one-token call of the single-launch kernel: stage 2 only)"""
+        return self.L.rq_w4a4_stage_mask(self.type, self.K, self.M, self.K)
+
+    def median_timed(self, steps, warmup, stages, batches=11):
         vals = sorted(self.timed(steps, warmup if b == 0 else 2, stages)[0] for b in range(batches))
         return vals[len(vals) // 2]
 
-    def check(self, oracle):
+    def check(self, oracle, want=None):
         import numpy as np
         self.call(3)
         self.torch.cuda.synchronize()
-        want = oracle.mul_mat(self.type, self.blocks, self.x_host, self.clip, n_rot=self.K)
+        if want is None:
+            want = oracle.mul_mat(self.type, self.blocks, self.x_host, self.clip, n_rot=self.K)
         got = self.y.cpu().numpy()
         return bool((got.view(np.uint32) == want.view(np.uint32)).all())
 
@@ -267,14 +277,26 @@ def cpu_baseline(oracle, prob, budget_s=12.0, max_reps=1500):   # about 20 core-
     return el / reps, reps, threads
 
 
+def cpu_one_pass(oracle, prob):
+    """one whole pass of the oracle over `prob` on the host's cores: (seconds, threads, result)"""
+    threads = min(host_cores()[1], 16)
+    t0 = time.perf_counter()
+    want = oracle.mul_mat(prob.type, prob.blocks, prob.x_host, prob.clip, n_rot=prob.K, n_threads=threads)
+    return time.perf_counter() - t0, threads, want
+
+
 def measure(prob, steps, warmup, bound):
     _, wall_ms = prob.timed(steps, warmup, 3)
     op_ms = prob.median_timed(steps, 2, 3)
     kern_ms = prob.median_timed(steps, warmup, 2)
-    act_ms = prob.median_timed(steps, warmup, 1)
+    # the activation side has launches of its own unless the single-launch kernel takes the call (then: null)
+    act_ms = prob.median_timed(steps, warmup, 1) if prob.stage_mask() & 1 else None
     K, N, M = prob.K, prob.N, prob.M
     out = {"K": K, "N": N, "M": M, "op_us": round(op_ms * 1e3, 3), "op_eager_wall_us": round(wall_ms * 1e3, 3),
-           "product_kernel_us": round(kern_ms * 1e3, 3), "activation_kernel_us": round(act_ms * 1e3, 3)}
+           "product_kernel_us": round(kern_ms * 1e3, 3),
+           "activation_kernel_us": None if act_ms is None else round(act_ms * 1e3, 3)}
+    if prob.type != prob.rq.TYPE_W4A4H:
+        out["type"] = "W4A4"
     if bound == "hbm":
         b = algorithmic_bytes(K, N, M)
         out.update(op_gbs=round(b / op_ms / 1e6, 1), kernel_gbs=round(b / kern_ms / 1e6, 1),
@@ -289,10 +311,10 @@ def measure(prob, steps, warmup, bound):
 
 
 def machine_peaks(torch, rq, code_bytes, batches=5):
-    """What plain probe kernels of the library reach on this machine, measured like the operator (graph-captured
-    batches between events): see rq_w4a4_probe in include/rq_w4a4.h."""
+    """What plain probe kernels reach on this machine, measured like the operator (graph-captured batches between
+    events): see rq_probe in include/rq_probe.h (librq_probe.so, a library of its own)."""
     import ctypes
-    L = rq.load_library()
+    L = rq.load_probe_library()
     dev = "cuda:0"
     cus = torch.cuda.get_device_properties(0).multi_processor_count
 
@@ -317,10 +339,10 @@ def machine_peaks(torch, rq, code_bytes, batches=5):
         return sorted(vals)[len(vals) // 2]
 
     def probe(buf, kind, a0, a1=0, a2=0, a3=0, off=0, nbytes=None):
-        rc = L.rq_w4a4_probe(kind, a0, a1, a2, a3, buf.data_ptr() + off, buf.numel() - off if nbytes is None else nbytes,
-                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        rc = L.rq_probe(kind, a0, a1, a2, a3, buf.data_ptr() + off, buf.numel() - off if nbytes is None else nbytes,
+                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
         if rc != 0:
-            raise RuntimeError("rq_w4a4_probe(%d) failed: %d" % (kind, rc))
+            raise RuntimeError("rq_probe(%d) failed: %d" % (kind, rc))
 
     out = {"compute_units": cus}
     small = torch.zeros(1 << 16, dtype=torch.uint8, device=dev)
@@ -350,8 +372,9 @@ def machine_peaks(torch, rq, code_bytes, batches=5):
     ops_per_mfma = 16 * 16 * 64 * 2
     mi, vi = 2000, 1000
 
-    def mix(sub, valu_op=0, one_wave_per_simd=False, m=mi, v=vi):
-        return timed(lambda i: probe(small, 2, sub | valu_op << 8 | (1 << 16 if one_wave_per_simd else 0), cus, m, v), 4)
+    def mix(sub, valu_op=0, one_wave_per_simd=False, m=mi, v=vi, form=0):
+        return timed(lambda i: probe(small, 2, sub | valu_op << 8 | (1 << 16 if one_wave_per_simd else 0) | form << 20,
+                                     cus, m, v), 4)
 
     simds = cus * 4
     t = mix(3)
@@ -359,7 +382,8 @@ def machine_peaks(torch, rq, code_bytes, batches=5):
     out["mfma_ns_per_instruction_per_simd"] = round(t * 1e3 / (mi * 16), 3)
     t = mix(0)
     out["mfma_i8_16x16x64_tops_two_wavefronts_per_simd"] = round(cus * 8 * mi * 16 * ops_per_mfma / t / 1e6, 1)
-    for op, name in ((0, "v_add_u32"), (1, "v_ashrrev_i32"), (2, "v_mul_i32_i24"), (3, "v_dot8c_i32_i4")):
+    for op, name in ((0, "v_add_u32"), (1, "v_ashrrev_i32"), (2, "v_mul_i32_i24"), (3, "v_dot8c_i32_i4"),
+                     (4, "v_fma_f32")):
         t1, t2 = mix(4, op), mix(1, op)
         out["valu_ns_per_instruction_per_simd_%s" % name] = {"one_wavefront": round(t1 * 1e3 / (vi * 128), 3),
                                                              "two_wavefronts": round(t2 * 1e3 / (2 * vi * 128), 3)}
@@ -377,6 +401,24 @@ def machine_peaks(torch, rq, code_bytes, batches=5):
     t = mix(5, 0, False, mi // 4, 0)
     out["same_wavefront_1_mfma_8_valu_ns_per_mfma_per_simd"] = round(t * 1e3 / (2 * (mi // 4) * 16), 3)
     out["same_wavefront_1_mfma_8_valu_tops"] = round(cus * 8 * (mi // 4) * 16 * ops_per_mfma / t / 1e6, 1)
+    # The other MFMA forms: alone (two wavefronts per SIMD), one MFMA wavefront beside one v_fma_f32 wavefront on every
+    # SIMD, and one wavefront interleaving each MFMA with 16 v_fma_f32 (what the fp6 GEMM's fold does per 32 x 32 tile
+    # and group). Ops per instruction: 32 x 32 x 32 x 2 (int8), 32 x 32 x 64 x 2 (f8f6f4).
+    forms = {}
+    m2 = mi // 4
+    for form, name, ops in ((1, "v_mfma_i32_32x32x32_i8", 65536), (2, "v_mfma_f32_32x32x64_f8f6f4_fp8", 131072),
+                            (3, "v_mfma_f32_32x32x64_f8f6f4_fp6", 131072)):
+        t_alone = mix(0, 4, False, m2, vi, form)
+        t_m, t_v, t_both = mix(3, 4, False, m2, vi, form), mix(4, 4, False, m2, vi, form), mix(2, 4, False, m2, vi, form)
+        t_16 = mix(6, 4, False, m2 // 2, 0, form)
+        forms[name] = {
+            "ns_per_instruction_per_simd": round(t_alone * 1e3 / (2 * m2 * 16), 3),
+            "tops": round(cus * 8 * m2 * 16 * ops / t_alone / 1e6, 1),
+            "beside_v_fma_f32_wavefront_us": {"mfma_alone": round(t_m, 1), "valu_alone": round(t_v, 1),
+                                              "together": round(t_both, 1), "sum": round(t_m + t_v, 1)},
+            "same_wavefront_1_mfma_16_v_fma_f32_ns_per_mfma_per_simd": round(t_16 * 1e3 / (2 * (m2 // 2) * 16), 3),
+            "same_wavefront_1_mfma_16_v_fma_f32_tops": round(cus * 8 * (m2 // 2) * 16 * ops / t_16 / 1e6, 1)}
+    out["mfma_forms"] = forms
     return out
 
 
@@ -435,9 +477,15 @@ def main():
         torch.cuda.empty_cache()
         extra["peaks"] = machine_peaks(torch, rq, N * K // 2)
     roofline_m2048 = None
+    cpu_m2048 = None
     if not args.no_extra:
+        W4A4 = rq.TYPE_W4A4
         shapes = [
+            # BASELINE config 1 (the reference's own CPU-runnable case): plain W4A4, no rotation
+            ("config1_w4a4_k4096_n1024_m1", 4096, 1024, 1, "normal", 1.0, "hbm", W4A4),
             ("decode_k5120_n5120_m1", 5120, 5120, 1, "outlier_channels", 0.9, "hbm"),
+            ("decode_k5120_n5120_m2", 5120, 5120, 2, "outlier_channels", 0.9, "hbm"),
+            ("decode_k5120_n5120_m4", 5120, 5120, 4, "outlier_channels", 0.9, "hbm"),
             ("decode_k5120_n5120_m8", 5120, 5120, 8, "outlier_channels", 0.9, "hbm"),
             ("down_k17408_n5120_m1", 17408, 5120, 1, "relu2", 1.0, "hbm"),
             ("down_k17408_n5120_m16", 17408, 5120, 16, "relu2", 1.0, "hbm"),
@@ -450,15 +498,17 @@ def main():
             ("perf_k5120_n6144_m8", 5120, 6144, 8, "normal", 1.0, "hbm"),
             ("perf_k5120_n6144_m16", 5120, 6144, 16, "normal", 1.0, "hbm"),
             ("perf_k5120_n6144_m512", 5120, 6144, 512, "normal", 1.0, "mfma"),
+            # the reference's perf mode times both types (patch lines 3067-3074): plain W4A4 on the largest weight
+            ("perf_w4a4_k5120_n17408_m1", 5120, 17408, 1, "normal", 1.0, "hbm", W4A4),
+            ("perf_w4a4_k5120_n17408_m512", 5120, 17408, 512, "normal", 1.0, "mfma", W4A4),
         ]
         want = [w for w in args.shapes.split(",") if w]
-        for name, k, n, m, kind, clip, bound in shapes:
+        for name, k, n, m, kind, clip, bound, *rest in shapes:
             if want and name not in want:
                 continue
             head = None
             torch.cuda.empty_cache()
-            head = None
-            head = Problem(k, n, m, kind, clip, seed=3)
+            head = Problem(k, n, m, kind, clip, seed=3, type_=rest[0] if rest else None)
             steps = args.steps if m <= 64 else max(20, args.steps // 10)
             extra[name], _, kms = measure(head, steps, min(args.warmup, steps), bound)
             if name == "prefill_k5120_n17408_m2048":
@@ -466,10 +516,23 @@ def main():
                 roofline_m2048 = {"bound": "mfma", "achieved": round(ops / kms / 1e9, 1), "peak": INT8_PEAK_TOPS,
                                   "unit": "TOP/s", "frac": round(ops / kms / 1e9 / INT8_PEAK_TOPS, 4),
                                   "traffic": profiled_traffic_bytes(GEMM_PROFILE, "traffic_bytes_per_launch_m2048:"),
-                                  "kernel": "rq_gemm_kernel (wide + narrow tiles of one launch)",
+                                  "kernel": "rq_gemm6_kernel<1> (fp6 MFMA; whole tiles and K slices of one launch)"
+                                            if os.environ.get("RQ_GEMM_FP6", "1") != "0" else "rq_gemm_kernel (int8 MFMA)",
                                   "kernel_us": round(kms * 1e3, 3), "workload": "W4A4H K=5120 N=17408 M=2048",
                                   "op_us": extra[name]["op_us"], "op_tops": extra[name]["op_tops"],
                                   "op_frac": extra[name]["op_frac_of_int8_peak"]}
+                if not args.no_cpu:
+                    # the CPU path beside the M = 2048 half of the metric: one whole pass of the oracle, whose result
+                    # is also what this problem's GPU output is compared with
+                    from oracle import rq_oracle
+                    sec, threads, want_y = cpu_one_pass(rq_oracle, head)
+                    nproc, usable = host_cores()
+                    cpu_m2048 = {"value": round(ops / sec / 1e12, 4), "unit": "TOP/s", "cores": threads, "nproc": nproc,
+                                 "cpus_usable": usable, "kind": "port",
+                                 "sample": "one whole-op pass of the same K=%d N=%d M=%d problem (%.2f s), CPU oracle, "
+                                           "two-phase threading" % (k, n, m, sec),
+                                 "parity_vs_oracle": head.check(rq_oracle, want_y)}
+                    del want_y
 
         for name, m in (("layer_m16", 16), ("layer_m1", 1)):
             if not want or name in want:
@@ -491,11 +554,12 @@ def main():
                      "frac": round(b / kern_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": profiled_traffic_bytes(),
                      # one token: rotation, quantizer, product and epilogue are ONE launch, so the dominant kernel
                      # is the whole operator (template arguments: Paley order, groups and remainder items in flight)
-                     "kernel": "rq_decode_kernel<20, 10, 4>" if res["activation_kernel_us"] < 1.0
+                     "kernel": "rq_decode_kernel<20, 10, 4>" if res["activation_kernel_us"] is None
                                else "rq_gemv_kernel<1, 4, 1>",
                      "kernel_us": round(kern_ms * 1e3, 3)},
         "roofline_m2048": roofline_m2048,
         "cpu_baseline": cpu,
+        "cpu_baseline_m2048": cpu_m2048,
         "parity_vs_oracle": parity,
         "extra": extra,
     }

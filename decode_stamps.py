@@ -3,15 +3,15 @@
 compute unit, taken by the first rotate wavefront and the first stream wavefront, kept in registers and written out
 when the kernel ends). Needs the instrumented build of the library: `make -C ruquant_amd/csrc stamps`.
 
-    python3 ruquant_amd/decode_stamps.py [K N]...        (default: the benchmark's one-token shapes)
+    python3 decode_stamps.py [K N]...        (default: the benchmark's one-token shapes)
 """
 import ctypes
 import os
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.dirname(HERE))
-os.environ["RQ_LIB_PATH"] = os.path.join(HERE, "lib", "librq_w4a4_stamps.so")
+sys.path.insert(0, HERE)
+os.environ["RQ_LIB_PATH"] = os.path.join(HERE, "ruquant_amd", "lib", "librq_w4a4_stamps.so")
 
 import torch  # noqa: E402
 import ruquant_amd as rq  # noqa: E402

@@ -201,26 +201,15 @@ int rq_w4a4_quantize_weights(int type, const float *w_dev, int64_t ldw, int64_t 
 int rq_w4a4_dequantize(int type, const void *blocks_dev, int64_t rows, int64_t K, int64_t n_rot, float *out_dev,
                        int64_t ldo, rq_stream_t stream);
 
-/* Measurement aid with no counterpart in the reference's operator (its method is the reference's
- * rig/membench/stream_bench.hip:1-60 and rig/bench_valu.cu:1-129): launches ONE machine-peak probe kernel on `stream`;
- * the caller times a batch of launches. buf: device scratch, 256-byte aligned, `bytes` long (>= 8192).
- *   RQ_PROBE_EMPTY : a0 workgroups of 256 threads that do nothing (cost of a launch).
- *   RQ_PROBE_STREAM: reads a0 bytes of buf with non-temporal 16-byte loads, a1 loads in flight per thread
- *                    (4, 5, 8, 10, 16 or 20), a2 workgroups (0: one per chunk of a1 * 4 KiB).
- *   RQ_PROBE_MIX   : a0 = sub-kind | VALU instruction << 8 | one-wavefront-per-SIMD << 16, a1 workgroups,
- *                    a2 MFMA iterations (16 v_mfma_i32_16x16x64_i8 each), a3 VALU iterations (128 instructions each).
- *                    Sub-kinds: 0 all wavefronts MFMA; 1 all VALU; 2 wavefronts 0..3 MFMA and 4..7 VALU (one of each
- *                    per SIMD); 3 wavefronts 0..3 MFMA, others idle; 4 wavefronts 4..7 VALU, others idle; 5 / 6 every
- *                    wavefront 1 MFMA + 8 / 16 VALU interleaved; 7 every wavefront its MFMAs, then its VALU work.
- *                    VALU instruction: 0 v_add_u32, 1 v_ashrrev_i32, 2 v_mul_i32_i24. The SIMD id each wavefront of
- *                    workgroup 0 ran on is written to the 8 ints at buf + 4096. */
-#define RQ_PROBE_EMPTY  0
-#define RQ_PROBE_STREAM 1
-#define RQ_PROBE_MIX    2
-int rq_w4a4_probe(int kind, int64_t a0, int64_t a1, int64_t a2, int64_t a3, void *buf, size_t bytes,
-                  rq_stream_t stream);
+/* Which stages of rq_w4a4_mul_mat_stages launch kernels for this problem: bit 0 = stage 1 (activation side), bit 1 =
+ * stage 2 (products). 2 for a one-token call that the single-launch kernel takes (stage 1 is then a no-op), 3
+ * otherwise, 0 for arguments the operator refuses. No counterpart in the reference (its act cache is internal,
+ * P:2163-2172); for hosts and benchmarks that time or capture the stages separately. */
+int rq_w4a4_stage_mask(int type, int64_t K, int64_t M, int64_t n_rot);
 
-/* Library version, for the host binding to check. */
+/* Library version, for the host binding to check: bumped whenever an entry point, an error code or the meaning of an
+ * argument changes. A binding built against this header refuses a library that reports another number. */
+#define RQ_ABI_VERSION 3
 int rq_w4a4_abi_version(void);
 
 #ifdef __cplusplus

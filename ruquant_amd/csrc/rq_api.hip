@@ -160,13 +160,14 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
     bool one_launch = false;
     if (n > 1) {
         const WorkspaceLayout Wsum = workspace_layout(K, Nsum, M);
-        if (ws_bytes >= Wsum.bytes) {
+        if (ws_bytes >= Wsum.bytes_min) {
             W = Wsum;
             one_launch = true;
         }
     }
     const int64_t Ncells = one_launch ? Nsum : Nmax;
-    if (ws_bytes < W.bytes || (reinterpret_cast<uintptr_t>(ws) & 255) != 0) return RQ_E_WORKSPACE;
+    if (ws_bytes < W.bytes_min || (reinterpret_cast<uintptr_t>(ws) & 255) != 0) return RQ_E_WORKSPACE;
+    const bool have_slabs = ws_bytes >= W.bytes;   // (fp6 GEMM: room to cut leftover tiles along K)
     uint8_t *wsb = reinterpret_cast<uint8_t *>(ws);
 
     // Activation groups of 128 / 256 (RQ_ACT_GROUP) change where the per-group floor falls. The GEMV and the skinny
@@ -307,7 +308,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             g.M = (int) M;
             g.Mp = (int) W.Mp;
             g.groups_per_fold = G / kGroup;
-            g.cells = wsb + W.off_tot;
+            g.cells = have_slabs ? wsb + W.off_tot : nullptr;
             e = fp6 ? launch_gemm6(g, stream) : launch_gemm(g, stream);
             if (e != hipSuccess) return (int) e;
         } else {
@@ -352,7 +353,7 @@ using namespace rq;
 
 extern "C" {
 
-int rq_w4a4_abi_version(void) { return 1; }
+int rq_w4a4_abi_version(void) { return RQ_ABI_VERSION; }
 
 int rq_w4a4_hadamard_factor(int64_t n, int *p, int *m) {
     int pp = 0, mm = 0;
@@ -438,7 +439,7 @@ int rq_w4a4_mul_mat(int type, const void *prepared_dev, int64_t K, int64_t N, co
 int rq_w4a4_mul_mat_static(int type, const void *prepared_dev, int64_t K, int64_t N, const float *x_dev, int64_t ldx,
                            int64_t M, float *y_dev, int64_t ldy, float clip, int64_t n_rot, rq_stream_t stream) {
     if (!shape_ok(type, K, N, M)) return RQ_E_UNSUPPORTED;
-    if (workspace_layout(K, N, M < 1 ? 1 : M).bytes > (size_t) RQ_STATIC_SCRATCH_BYTES) return RQ_E_LIMIT;
+    if (workspace_layout(K, N, M < 1 ? 1 : M).bytes_min > (size_t) RQ_STATIC_SCRATCH_BYTES) return RQ_E_LIMIT;
     hipError_t e = hipSuccess;
     void *ws = static_scratch(&e);   // resolved by rq_w4a4_prepare on this device; here only looked up
     if (!ws) return (int) e;
@@ -452,6 +453,15 @@ int rq_w4a4_mul_mat_stages(int type, const void *prepared_dev, int64_t K, int64_
     if (stages < 1 || stages > 3) return RQ_E_ARGUMENT;
     return run_products(type, 1, &prepared_dev, K, &N, x_dev, ldx, M, &y_dev, &ldy, clip, n_rot, workspace_dev,
                         workspace_bytes, (hipStream_t) stream, stages);
+}
+
+int rq_w4a4_stage_mask(int type, int64_t K, int64_t M, int64_t n_rot) {
+    if (!is_w_type(type) || K <= 0 || K % RQ_BLOCK_CODES != 0 || K > RQ_MAX_K || M < 1) return 0;
+    int p, m;
+    if (!rotation_of(type, K, n_rot, p, m)) return 0;
+    // one token that the single-launch kernel takes: everything happens in stage 2
+    if (M == 1 && env().decode_fused && decode_takes((int) K, type == RQ_TYPE_W4A4H, p, m, env().act_group)) return 2;
+    return 3;
 }
 
 int rq_w4a4_mul_mat_fused(int type, int n, const void *const *prepared_dev, int64_t K, const int64_t *N,

@@ -99,14 +99,18 @@ inline size_t act6_plane_bytes(int ng, int64_t Mp) { return (size_t) ng * (size_
 //   cells  : split-K cells [8 or 64 tokens][n_panels * 64], 64 bits each: arrival count above bit 48, exact sum
 //            below.
 // ---------------------------------------------------------------------------------------------------
+constexpr int kPlanUnits = 256;   // compute units the fp6 GEMM's launch plan counts with (MI355X)
+constexpr size_t kGemm6CounterBytes = kPlanUnits * sizeof(int32_t);
+constexpr size_t kGemm6ScratchBytes = kGemm6CounterBytes + (size_t) kPlanUnits * 256 * 128 * sizeof(int32_t);
+
 struct WorkspaceLayout {
     int64_t Mp;       // tokens padded to the GEMM tile
     int     chunks;   // ceil(M / 8)
     size_t  off_u, off_act, off_lohi, off_rpart, off_i8, off_tot, bytes;
     size_t  tot_ints;   // ints of the split-K cells at off_tot (two per cell)
+    size_t  bytes_min;  // what a call needs at the least: `bytes` without the slabs of the fp6 GEMM's K slices (a
+                        // workspace between the two runs every tile whole)
 };
-
-size_t gemm6_cell_bytes_max(int64_t N, int64_t M, int ng);
 
 inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
     WorkspaceLayout W;
@@ -130,14 +134,14 @@ inline WorkspaceLayout workspace_layout(int64_t K, int64_t N, int64_t M) {
     W.off_i8 = small ? off + gemv_form : off;
     off = align_up(off + (small ? gemv_form + act_i8 : act_i8), 256);
     W.tot_ints = (size_t) 2 * (M <= kGemvTokens ? kGemvTokens : kSkinnyTokens) * n_panels * kPanelRows;
-    if (M > kSkinnyTokens && gemm_fp6_enabled()) {
-        // the fp6 GEMM's arrival cells (the tiles it cuts along K); sized for the widest activation group's plan, which
-        // cuts the most
-        const size_t cb = gemm6_cell_bytes_max(N, M, ng);
-        if (cb / sizeof(int32_t) > W.tot_ints) W.tot_ints = cb / sizeof(int32_t);
-    }
     W.off_tot = off;
     off = align_up(off + W.tot_ints * sizeof(int32_t), 256);
+    W.bytes_min = off;
+    if (M > kSkinnyTokens && gemm_fp6_enabled() && kGemm6ScratchBytes > W.tot_ints * sizeof(int32_t)) {
+        // the fp6 GEMM's arrival counters and slabs for the tiles it cuts along K: never more than kPlanUnits slices
+        // (a constant, so that the workspace grows monotonically with the token count)
+        off = align_up(W.off_tot + kGemm6ScratchBytes, 256);
+    }
     W.bytes = off;
     return W;
 }
@@ -267,8 +271,7 @@ hipError_t launch_gemm6(const GemmArgs &a, hipStream_t stream);
 // How a launch of the fp6 form is cut: n_whole tiles (256 rows x 128 tokens) run whole, the rest in `parts` slices of
 // K each, which meet in cell_bytes of workspace: kGemm6CounterBytes of arrival counters (one int per cut tile: zero on
 // entry, left zero), then one slab of partial totals per slice (needs no clearing).
-constexpr int kPlanUnits = 256;
-constexpr size_t kGemm6CounterBytes = kPlanUnits * sizeof(int32_t);
+
 struct Gemm6Plan {
     int    n_tiles, n_whole, parts;
     size_t cell_bytes;

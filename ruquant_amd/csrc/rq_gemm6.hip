@@ -34,6 +34,10 @@
 
 #pragma clang fp contract(off)
 
+#ifndef RQ6_VARIANT
+#define RQ6_VARIANT 0
+#endif
+
 namespace rq {
 
 namespace {
@@ -345,6 +349,10 @@ __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, 
                                        int32_t (&tot)[2][2][16]) {
     Stage *ring[kRing] = { &s0, &s1, &s2, &s3 };
     Operands X, Y;
+    if (RQ6_VARIANT == 3 || RQ6_VARIANT == 5) {
+        for (int i = 0; i < 2; ++i) for (int e = 0; e < 6; ++e) { X.A[i][e] = c.lane * (e + 1); X.B[i][e] = c.lane * (e + i + 3); Y.A[i][e] = c.lane * (e + 7); Y.B[i][e] = c.lane * (e + i + 2); }
+        X.m4[0] = X.m4[1] = Y.m4[0] = Y.m4[1] = 4.0f;
+    }
     v16f P = {};
     float pm = 0.0f;
     fetch(c, s0, 0);
@@ -362,16 +370,16 @@ __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, 
             const Stage &cur = *ring[j];
             const Stage &next = *ring[(j + 1) % kRing];
             Stage &refill = *ring[(j + 3) % kRing];
-            read_operands(c, cur, 1, Y);
+            if (RQ6_VARIANT != 3 && RQ6_VARIANT != 5) read_operands(c, cur, 1, Y);
             __builtin_amdgcn_sched_barrier(0);
             group_units<HASK>(c, X, c.g0 + 2 * st, P, pm, acc, tot);
             // stage st + 1 is whole once every wavefront has seen its own loads of it arrive (those of step st + 2
             // may still be in flight); stage st - 1 is then free for step st + 3
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerStep) : "memory");
-            __builtin_amdgcn_s_barrier();
+            if (RQ6_VARIANT != 4 && RQ6_VARIANT != 5 && RQ6_VARIANT != 6) __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            fetch(c, refill, st + 3);
-            read_operands(c, next, 0, X);   // (past the last step: stale cells, never used)
+            if (RQ6_VARIANT != 1 && RQ6_VARIANT != 5 && RQ6_VARIANT != 7) fetch(c, refill, st + 3);
+            if (RQ6_VARIANT != 3 && RQ6_VARIANT != 5) read_operands(c, next, 0, X);   // (past the last step: stale cells, never used)
             __builtin_amdgcn_sched_barrier(0);
             group_units<HASK>(c, Y, c.g0 + 2 * st + 1, P, pm, acc, tot);
         }
@@ -652,15 +660,22 @@ Gemm6Plan gemm6_plan(int64_t N, int64_t M, int ng, int groups_per_fold) {
     // not depend on the device, because the workspace is sized from it.)
     const int left = pl.n_tiles % kPlanUnits;
     if (left > 0 && kPlanUnits / left >= 2) {
-        int parts = kPlanUnits / left;
+        // more slices = less work per slice, but the workgroup that completes a tile reads the other slices' slabs one
+        // after the other (about 2 us each) and every slice pays its own start (about 5 us): per step 1.1 us
         const int steps = ng / 2;
-        if (parts > steps / 2) parts = steps / 2;               // at least two steps per slice
-        // wider activation groups: a slice holds whole groups and an even number of steps
-        if (groups_per_fold > 1) {
-            while (parts > 1 && steps % (2 * parts) != 0) --parts;
+        int best = 1;
+        double best_cost = 1.1 * steps;
+        for (int parts = 2; parts <= kPlanUnits / left && parts <= steps / 2; ++parts) {
+            // wider activation groups: a slice holds whole groups and an even number of steps
+            if (groups_per_fold > 1 && steps % (2 * parts) != 0) continue;
+            const double cost = 1.1 * ((steps + parts - 1) / parts) + 5.0 + 2.0 * (parts - 1);
+            if (cost < best_cost) {
+                best_cost = cost;
+                best = parts;
+            }
         }
-        if (parts >= 2) {
-            pl.parts = parts;
+        if (best >= 2) {   // (left * parts <= kPlanUnits slices: the workspace holds a slab for each)
+            pl.parts = best;
             pl.n_whole = pl.n_tiles - left;
         }
     }
@@ -669,21 +684,16 @@ Gemm6Plan gemm6_plan(int64_t N, int64_t M, int ng, int groups_per_fold) {
     return pl;
 }
 
-size_t gemm6_cell_bytes_max(int64_t N, int64_t M, int ng) {
-    size_t best = 0;
-    for (int gf = 1; gf <= 4; gf *= 2) {
-        const size_t b = gemm6_plan(N, M, ng, gf).cell_bytes;
-        if (b > best) best = b;
-    }
-    return best;
-}
-
 hipError_t launch_gemm6(const GemmArgs &a, hipStream_t stream) {
     const uint8_t *p = a.prepared;
     const int n_row_tiles = a.L.n_rtiles;
     const int n_tok_tiles = a.Mp / kTileTok;
-    const Gemm6Plan pl = gemm6_plan(a.L.N, a.M, a.L.ng, a.groups_per_fold);
-    if (pl.n_tiles != n_row_tiles * n_tok_tiles || (pl.parts > 1 && a.cells == nullptr)) return hipErrorInvalidValue;
+    Gemm6Plan pl = gemm6_plan(a.L.N, a.M, a.L.ng, a.groups_per_fold);
+    if (pl.n_tiles != n_row_tiles * n_tok_tiles) return hipErrorInvalidValue;
+    if (a.cells == nullptr) {   // a workspace without slabs: every tile whole
+        pl.n_whole = pl.n_tiles;
+        pl.parts = 1;
+    }
     const int super_tiles = n_tok_tiles % 4 == 0 && n_row_tiles % 8 == 0;
     const int grid = pl.n_whole + (pl.n_tiles - pl.n_whole) * pl.parts;
     const float *m4 = reinterpret_cast<const float *>(a.act8 + act6_plane_bytes(a.L.ng, a.Mp));

@@ -74,6 +74,9 @@ size_t workspace_for(int type, int64_t K, int64_t N, int64_t max_tokens) {
 // first use, never inside a graph capture: read block 0's header, resolve clip and rotation length, prepare
 rq_first_use *first_use(rq_backend_context &ctx, const rq_tensor *src0) {
     if (src0->extra) return (rq_first_use *) src0->extra;
+    if (rq_w4a4_abi_version() != RQ_ABI_VERSION) {
+        rq_abort("librq_w4a4.so is not the version this adapter was built against", rq_w4a4_abi_version(), RQ_ABI_VERSION);
+    }
     rq_block_w4a4 hdr;
     hipStream_t stream = (hipStream_t) ctx.stream;
     hip_check(hipMemcpyAsync(&hdr, src0->data, 16, hipMemcpyDeviceToHost, stream), "header read");

@@ -14,10 +14,9 @@ class LibraryMissing(RuntimeError):
 
 
 def build_library(jobs=8):
-    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU): the library, the host program and the
-    instrumented build of the decode kernel that ruquant_amd/decode_stamps.py loads."""
+    """Compile every HIP source for gfx950 (hipcc cross-compiles without a GPU): the operator's library, the host
+    program and the probe library of the benchmark."""
     subprocess.run(["make", "-C", CSRC, "-B", "-j%d" % jobs, "all"], check=True)
-    subprocess.run(["make", "-C", CSRC, "stamps"], check=True)
     return LIB_PATH
 
 
@@ -26,6 +25,8 @@ _lib = None
 c_f32p = ctypes.POINTER(ctypes.c_float)
 c_i64p = ctypes.POINTER(ctypes.c_int64)
 c_intp = ctypes.POINTER(ctypes.c_int)
+
+ABI_VERSION = 3   # RQ_ABI_VERSION of include/rq_w4a4.h
 
 PROTOTYPES = {
     "rq_w4a4_abi_version": (ctypes.c_int, []),
@@ -71,8 +72,7 @@ PROTOTYPES = {
                                                 ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "rq_w4a4_dequantize": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
                                           ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
-    "rq_w4a4_probe": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
-                                     ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "rq_w4a4_stage_mask": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64]),
     "rq_w4a4_quantize_act": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
                                             ctypes.c_int64, ctypes.c_float, ctypes.c_int64, ctypes.c_void_p,
                                             ctypes.c_void_p]),
@@ -88,9 +88,35 @@ def load_library():
                 "%s is missing: build it with `make -C %s` (or __graft_entry__.build()); there is no fallback path"
                 % (LIB_PATH, CSRC))
         L = ctypes.CDLL(LIB_PATH)
+        try:
+            L.rq_w4a4_abi_version.restype = ctypes.c_int
+            version = L.rq_w4a4_abi_version()
+        except AttributeError:
+            version = None
+        if version != ABI_VERSION:
+            raise LibraryMissing("%s reports ABI version %s, this binding is written for %d: rebuild it with `make -C %s`"
+                                 % (LIB_PATH, version, ABI_VERSION, CSRC))
         for name, (res, args) in PROTOTYPES.items():
             fn = getattr(L, name)
             fn.restype = res
             fn.argtypes = args
         _lib = L
     return _lib
+
+
+PROBE_PATH = os.path.join(_HERE, "lib", "librq_probe.so")
+_probe = None
+
+
+def load_probe_library():
+    """ctypes handle of librq_probe.so (include/rq_probe.h): the machine-peak probe kernels of the benchmark."""
+    global _probe
+    if _probe is None:
+        if not os.path.exists(PROBE_PATH):
+            raise LibraryMissing("%s is missing: build it with `make -C %s`" % (PROBE_PATH, CSRC))
+        P = ctypes.CDLL(PROBE_PATH)
+        P.rq_probe.restype = ctypes.c_int
+        P.rq_probe.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                               ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        _probe = P
+    return _probe

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import ruquant_amd as rq
-from ruquant_amd.lib import PROTOTYPES, LIB_PATH
+from ruquant_amd.lib import PROTOTYPES, LIB_PATH, ABI_VERSION, PROBE_PATH
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -27,7 +27,31 @@ def test_library_exports_every_declared_symbol():
     for s in syms:
         assert hasattr(L, s), s
         assert s in PROTOTYPES, "python binding lacks %s" % s
-    assert L.rq_w4a4_abi_version() == 1
+    assert L.rq_w4a4_abi_version() == ABI_VERSION
+    header = open(os.path.join(ROOT, "include", "rq_w4a4.h")).read()
+    assert int(re.search(r"#define RQ_ABI_VERSION (\d+)", header).group(1)) == ABI_VERSION
+
+
+def test_probe_library_exports_its_header():
+    text = open(os.path.join(ROOT, "include", "rq_probe.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    syms = sorted(set(re.findall(r"\b(rq_probe\w*)\s*\(", text)))
+    assert syms == ["rq_probe"]
+    P = rq.load_probe_library()
+    assert hasattr(P, "rq_probe")
+    assert os.path.exists(PROBE_PATH) and PROBE_PATH.startswith(ROOT)
+    # the operator's library carries no measurement kernels
+    assert not hasattr(rq.load_library(), "rq_probe") and not hasattr(rq.load_library(), "rq_w4a4_probe")
+
+
+def test_stage_mask_is_a_host_query():
+    L = rq.load_library()
+    assert L.rq_w4a4_stage_mask(rq.TYPE_W4A4H, 5120, 1, 5120) in (2, 3)   # (3 under RQ_DECODE_FUSED=0 / RQ_ACT_GROUP)
+    assert L.rq_w4a4_stage_mask(rq.TYPE_W4A4H, 17408, 1, 17408) == 3       # H68: two launches at one token
+    assert L.rq_w4a4_stage_mask(rq.TYPE_W4A4H, 5120, 2, 5120) == 3
+    assert L.rq_w4a4_stage_mask(rq.TYPE_W4A4, 4096, 512, 4096) == 3
+    assert L.rq_w4a4_stage_mask(12, 4096, 1, 4096) == 0
+    assert L.rq_w4a4_stage_mask(rq.TYPE_W4A4H, 5120, 1, 1000) == 0
 
 
 def test_library_is_in_tree():
