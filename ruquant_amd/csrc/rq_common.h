@@ -17,10 +17,9 @@ constexpr int kGemmTokens = 128;  // token tile of the MFMA GEMM; int8 activatio
 constexpr int kRangeParts = 32;    // partial maxima of a token's group ranges handed from the activation kernel to the GEMV
 constexpr int kSkinnyTokens = 64;   // most tokens of one pass of the skinny MFMA kernel
 constexpr int kTwoStepTokens = 40;   // long Paley stages: most tokens whose rotation is spread over several workgroups each
-constexpr int kGemvWideTokens = 8;   // most tokens of a GEMV pass with activation groups of 128 / 256
 constexpr int kGemvMaxTokens = 64;  // workspaces of up to this many tokens hold the fp32 form too (the GEMV takes up to 4
-                                    // tokens, up to 8 with activation groups of 128 / 256; the skinny path's two-step
-                                    // activation side uses the fp32 rows as an intermediate)
+                                    // tokens whatever the activation group; the skinny path's two-step activation
+                                    // side, 5 .. 40 tokens, uses the fp32 rows as an intermediate)
 
 // ---------------------------------------------------------------------------------------------------
 // Prepared weight (written once by rq_w4a4_prepare, read by every product kernel).
@@ -88,7 +87,7 @@ inline size_t act6_plane_bytes(int ng, int64_t Mp) { return (size_t) ng * (size_
 // Workspace of one rq_w4a4_mul_mat call.
 //
 //   u      : Mp floats, the token units (GEMM path; the GEMV derives them itself).
-//   act    : GEMV path (M <= 4; M <= 8 with wide activation groups): the rotated activations as fp32 rows [M][K] followed by the clipped group
+//   act    : GEMV path (M <= 4): the rotated activations as fp32 rows [M][K] followed by the clipped group
 //            ranges [M][ng][2] (lo, hi) and [M][32] partial maxima of hi - lo; every GEMV workgroup quantizes
 //            the K slice it consumes itself.
 //            MFMA paths: two int8 digit planes of m (q - z), [g][digit][quarter][Mp][16 bytes], in the byte order
@@ -247,8 +246,8 @@ struct GemvArgs {
     int64_t         ldx;    // row stride in floats
     const float    *lohi;   // clipped group ranges of this chunk's first token, [T][ng][2]
     const float    *rpart;  // partial range maxima of this chunk's first token, [T][kRangeParts]
-    int             T;      // 1..8 tokens
-    int             gf;     // runs of 64 per activation group: 1, or 2 / 4 under RQ_ACT_GROUP (then T <= kGemvWideTokens)
+    int             T;      // 1..4 tokens
+    int             gf;     // runs of 64 per activation group: 1, or 2 / 4 under RQ_ACT_GROUP
     int32_t        *tot;    // split-K cells (zero on entry, left zero)
 };
 hipError_t launch_gemv(const GemvArgs &a, hipStream_t stream);

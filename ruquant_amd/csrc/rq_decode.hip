@@ -106,10 +106,12 @@ __device__ __forceinline__ void wait_count(const int *cnt, int target) {
 // (The add needs no wait for the wavefront's LDS writes in front of it: a wavefront's LDS instructions are carried out in
 // the order of issue, so whoever sees the count sees the writes. It returns the count, and the wavefront that
 // arrives last, the one the others wait for, knows so from the answer and does not poll: two LDS round trips less on
-// the critical path of every phase.)
+// the critical path of every phase. The ordering rests on that in-order LDS queue plus the compiler barrier in front of
+// the add, which keeps the compiler from sinking the phase's plain LDS stores below the relaxed atomic.)
 __device__ __forceinline__ void rot_sync(int *cnt, int &target, int lane) {
     target += kRotWaves;
     int seen = 0;
+    asm volatile("" ::: "memory");
     if (lane == 0) seen = atomicAdd(cnt, 1) + 1;
     seen = __builtin_amdgcn_readfirstlane(seen);
     if (seen < target) wait_count<false>(cnt, target);

@@ -326,11 +326,9 @@ hipError_t launch_twg(const GemvArgs &a, int nks, hipStream_t stream) {
 
 template <int T>
 hipError_t launch_t(const GemvArgs &a, int nks, hipStream_t stream) {
-    if constexpr (T <= kGemvWideTokens) {
-        // activation groups of 128 / 256 (a format variant): one configuration
-        if (a.gf == 2) return launch_twg<T, kGemvWaves, 2>(a, nks, stream);
-        if (a.gf == 4) return launch_twg<T, kGemvWaves, 4>(a, nks, stream);
-    }
+    // activation groups of 128 / 256 (a format variant): one configuration
+    if (a.gf == 2) return launch_twg<T, kGemvWaves, 2>(a, nks, stream);
+    if (a.gf == 4) return launch_twg<T, kGemvWaves, 4>(a, nks, stream);
     if (a.gf != 1) return hipErrorInvalidValue;
     return launch_twg<T, kGemvWaves, 1>(a, nks, stream);
 }
@@ -375,11 +373,7 @@ hipError_t launch_gemv(const GemvArgs &a, hipStream_t stream) {
         case 2: return launch_t<2>(a, nks, stream);
         case 3: return launch_t<3>(a, nks, stream);
         case 4: return launch_t<4>(a, nks, stream);
-        case 5: return launch_t<5>(a, nks, stream);
-        case 6: return launch_t<6>(a, nks, stream);
-        case 7: return launch_t<7>(a, nks, stream);
-        case 8: return launch_t<8>(a, nks, stream);
-        default: return hipErrorInvalidValue;
+        default: return hipErrorInvalidValue;   // (the dispatcher sends five tokens and more to the MFMA kernels)
     }
 }
 

@@ -33,9 +33,9 @@ for type_, N, K, wgroup in cases:
             print("wgroup=64 refused: %s" % e, flush=True)
         continue
     W = rq.W4A4Weight(blocks, type_, DEV)
-    # up to eight tokens the GEMV folds the wide groups, up to 64 the skinny MFMA kernel (one or two token tiles per
-    # wavefront, blocks of 32 tokens), beyond that the narrow-tile GEMM
-    for M in (1, 2, 3, 5, 8, 9, 16, 17, 32, 33, 40, 64, 65, 130):
+    # up to four tokens the GEMV folds the wide groups, from five to 64 the skinny MFMA kernel (one or two token tiles
+    # per wavefront, blocks of 32 tokens), beyond that the fp6 GEMM, whose MFMAs of a group chain through the accumulator
+    for M in (1, 2, 3, 5, 8, 9, 16, 17, 32, 33, 40, 64, 65, 130, 300):
         x = adversarial_activations(M, K, type_, wf, seed=M)
         got = run_gpu(W, x)
         want = rq_oracle.mul_mat(type_, blocks, x, W.clip, n_rot=max(W.n_rot, 0), G=G)

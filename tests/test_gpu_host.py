@@ -93,3 +93,60 @@ def test_host_reports_unsupported_shape(tmp_path):
     x = synth.activations("normal", M, K, 2)
     r, _ = _run(tmp_path, type_, K, N, M, blocks, x)
     assert r.returncode == 3 and json.loads(r.stdout.strip())["supported"] is False
+
+
+@pytest.mark.gpu
+def test_python_shared_activation_layer_chain(oracle):
+    """SharedActivation (the Python host's counterpart of the reference's rq_act_cache, patch lines 1996-2023,
+    2163-2172) over one transformer layer's seven products in the layer's dataflow: q, k, v share one quantized x,
+    gate and up another. Every output equals the oracle's bits; hits and misses are counted. Orders in which the
+    second weight of a shared x is the larger one (k before q, up after a smaller gate stand-in) must miss again
+    where the split-K cells of the first call do not cover its rows."""
+    import numpy as np
+    import torch
+    import ruquant_amd as rq
+    from ruquant_amd import synth
+    from tests.gpu_util import bits_equal, first_mismatch
+
+    dev = "cuda:0"
+    type_ = rq.TYPE_W4A4H
+    shapes = {"q": (5120, 1536), "k": (5120, 256), "v": (5120, 256), "o": (1536, 5120), "gate": (5120, 2176),
+              "up": (5120, 2176), "down": (2176 * 2, 5120)}
+    shapes["down"] = (4352, 5120)     # 68 x 64: the long Paley stage
+    shapes["gate"] = shapes["up"] = (5120, 4352)
+    blocks = {n: synth.random_weight_blocks(N, K, 50 + i, type_, clip=0.0) for i, (n, (K, N)) in enumerate(shapes.items())}
+    W = {n: rq.W4A4Weight(blocks[n], type_, dev) for n in shapes}
+    L = rq.load_library()
+    for M in (1, 3, 16, 40, 70):
+        x0 = synth.activations("normal", M, 5120, 60 + M)
+        ws = torch.empty(max(L.rq_w4a4_workspace_bytes(type_, K, N, M) for K, N in shapes.values()), dtype=torch.uint8,
+                         device=dev)
+        sa = rq.SharedActivation(ws)
+        out = {n: torch.full((M, N), float("nan"), dtype=torch.float32, device=dev) for n, (K, N) in shapes.items()}
+        xd = torch.from_numpy(x0).to(dev)
+        for order in (("q", "k", "v"), ("k", "q", "v")):
+            sa.begin()
+            h0, m0 = sa.hits, sa.misses
+            for n in order:
+                sa.mul_mat(W[n], xd, out[n])
+            # one miss for the first weight; a later, larger weight misses again when the cells cleared for the first
+            # do not cover its rows (k before q), everything else hits
+            expect_miss = 1 if order[0] == "q" else 2
+            assert (sa.misses - m0, sa.hits - h0) == (expect_miss, 3 - expect_miss), (M, order, sa.misses - m0)
+            torch.cuda.synchronize()
+            ref = {n: oracle.mul_mat(type_, blocks[n], x0, 1.0, n_rot=5120) for n in ("q", "k", "v")}
+            for n in order:
+                got = out[n].cpu().numpy()
+                assert bits_equal(got, ref[n]), "M=%d order=%s %s: %s" % (M, order, n, first_mismatch(got, ref[n]))
+        sa.mul_mat(W["o"], out["q"], out["o"])
+        sa.mul_mat(W["gate"], out["o"], out["gate"])
+        sa.mul_mat(W["up"], out["o"], out["up"])
+        sa.mul_mat(W["down"], out["up"], out["down"])
+        torch.cuda.synchronize()
+        ro = oracle.mul_mat(type_, blocks["o"], ref["q"], 1.0, n_rot=1536)
+        rg = oracle.mul_mat(type_, blocks["gate"], ro, 1.0, n_rot=5120)
+        ru = oracle.mul_mat(type_, blocks["up"], ro, 1.0, n_rot=5120)
+        rd = oracle.mul_mat(type_, blocks["down"], ru, 1.0, n_rot=4352)
+        for n, r in (("o", ro), ("gate", rg), ("up", ru), ("down", rd)):
+            got = out[n].cpu().numpy()
+            assert bits_equal(got, r), "M=%d %s: %s" % (M, n, first_mismatch(got, r))

@@ -45,7 +45,8 @@ PAIRS = [
     ((rq.TYPE_W4A4H, 5120, 1024, 48), (rq.TYPE_W4A4H, 5120, 1024, 5)),      # skinny MFMA kernel, fewer tokens
     ((rq.TYPE_W4A4H, 6144, 512, 200), (rq.TYPE_W4A4, 512, 136, 17)),        # tiled GEMM, then skinny on another type
     ((rq.TYPE_W4A4H, 17408, 320, 16), (rq.TYPE_W4A4H, 17408, 320, 2)),      # two-step activation side, then GEMV
-    ((rq.TYPE_W4A4, 4096, 1024, 130), (rq.TYPE_W4A4, 4096, 1024, 1)),       # GEMM leaves digit planes where cells go
+    ((rq.TYPE_W4A4, 4096, 1024, 130), (rq.TYPE_W4A4, 4096, 1024, 3)),       # GEMM leaves its planes where the GEMV's cells go
+    ((rq.TYPE_W4A4H, 2560, 2048, 300), (rq.TYPE_W4A4H, 2560, 2048, 9)),     # the same in front of the skinny kernel's cells
 ]
 
 
@@ -61,6 +62,46 @@ def test_static_workspace_matches_caller_workspace(oracle, first, second):
         if i == 1:
             ref = oracle.mul_mat(type_, blocks, x_np, W.clip, n_rot=max(W.n_rot, 0))
             assert bits_equal(got, ref), "call 2 vs the CPU oracle: %s" % first_mismatch(got, ref)
+
+
+def test_static_call_allocates_nothing_and_can_be_captured(oracle):
+    """Free device memory is the same before and after eager calls, and a HIP graph that holds static calls of the three
+    small-batch paths (1, 3 and 16 tokens; capture forbids allocation) replays to the oracle's bits every time."""
+    L = rq.load_library()
+    type_, K, N = rq.TYPE_W4A4H, 5120, 1088
+    blocks = synth.random_weight_blocks(N, K, 31, type_, clip=0.9)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    probs = []
+    for M in (1, 3, 16):
+        x_np = synth.activations("outlier_channels", M, K, 40 + M)
+        probs.append((M, x_np, torch.from_numpy(x_np).to(DEV), torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)))
+
+    def run_all():
+        for M, _, x, y in probs:
+            rc = L.rq_w4a4_mul_mat_static(type_, W.prepared.data_ptr(), K, N, x.data_ptr(), K, M, y.data_ptr(), N, W.clip,
+                                          K, _stream())
+            assert rc == 0, rc
+
+    run_all()
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        run_all()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    want = [oracle.mul_mat(type_, blocks, x_np, W.clip, n_rot=K) for _, x_np, _, _ in probs]
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        run_all()
+    for replay in range(3):
+        for _, _, _, y in probs:
+            y.fill_(float("nan"))          # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for (M, _, _, y), ref in zip(probs, want):
+            got = y.cpu().numpy()
+            assert bits_equal(got, ref), "replay %d, M=%d: %s" % (replay, M, first_mismatch(got, ref))
 
 
 def test_static_workspace_refuses_what_does_not_fit():
