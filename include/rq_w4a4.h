@@ -88,6 +88,19 @@ size_t rq_w4a4_prepared_bytes(int64_t K, int64_t N);
 int rq_w4a4_prepare(const void *w_blocks_dev, int64_t K, int64_t N,
                     void *prepared_dev, size_t prepared_bytes, rq_stream_t stream);
 
+/* The same rewrite IN PLACE, as the reference does it (rq_repack_once, P:2046-2075): afterwards w_blocks_dev is the
+ * prepared weight (pass it as prepared_dev) and no longer readable as blocks, so one copy of the codes is resident
+ * instead of two. The codes, row scales, multipliers and flag word take 33 bytes per 64 codes against the blocks' 36
+ * and so fit where the blocks were (RQ_E_WORKSPACE for the few tiny shapes where the padding to 64 rows does not). The
+ * fp6 plane of the wide-batch kernel does not fit there: it goes to plane6_dev, rq_w4a4_plane6_bytes(K, N) bytes that
+ * the caller owns for as long as the weight is used (0 bytes and a null pointer under RQ_GEMM_FP6=0). staging_dev: at
+ * least rq_w4a4_inplace_staging_bytes(K, N) of scratch, free again when the stream has passed this call (a
+ * workspace will do). w_blocks_dev, plane6_dev and staging_dev 256-byte aligned. First use only: not graph-safe. */
+size_t rq_w4a4_plane6_bytes(int64_t K, int64_t N);
+size_t rq_w4a4_inplace_staging_bytes(int64_t K, int64_t N);
+int rq_w4a4_prepare_inplace(void *w_blocks_dev, int64_t K, int64_t N, void *plane6_dev, size_t plane6_bytes,
+                            void *staging_dev, size_t staging_bytes, rq_stream_t stream);
+
 /* ---- steady state --------------------------------------------------------------------------------- */
 
 /* Scratch the op needs for this problem (quantized activations, multipliers, split-K sums); a multiple of

@@ -424,6 +424,43 @@ int rq_w4a4_prepare(const void *w_blocks_dev, int64_t K, int64_t N, void *prepar
     return (int) launch_prepare(w_blocks_dev, L, reinterpret_cast<uint8_t *>(prepared_dev), (hipStream_t) stream);
 }
 
+size_t rq_w4a4_plane6_bytes(int64_t K, int64_t N) {
+    if (K <= 0 || K % RQ_BLOCK_CODES != 0 || K > RQ_MAX_K || N <= 0 || !gemm_fp6_enabled()) return 0;
+    const PreparedLayout L = prepared_layout(K, N);
+    return L.bytes - L.off_w6;
+}
+
+size_t rq_w4a4_inplace_staging_bytes(int64_t K, int64_t N) {
+    if (K <= 0 || K % RQ_BLOCK_CODES != 0 || K > RQ_MAX_K || N <= 0) return 0;
+    const PreparedLayout L = prepared_layout(K, N);
+    // the least, plus room for chunks of 32 panels (fewer launches)
+    return align_up(inplace_staging_min(L) + (size_t) 31 * kPanelRows * (L.ng / 4) * RQ_BLOCK_BYTES, 256);
+}
+
+int rq_w4a4_prepare_inplace(void *w_blocks_dev, int64_t K, int64_t N, void *plane6_dev, size_t plane6_bytes,
+                            void *staging_dev, size_t staging_bytes, rq_stream_t stream) {
+    if (!w_blocks_dev || !staging_dev) return RQ_E_ARGUMENT;
+    if (K <= 0 || K % RQ_BLOCK_CODES != 0 || K > RQ_MAX_K || N <= 0 || N > (int64_t) 1 << 24) return RQ_E_UNSUPPORTED;
+    const PreparedLayout L = prepared_layout(K, N);
+    // the sections up to the flag word must fit where the blocks are
+    if (L.off_flags + 256 > (size_t) N * (size_t) (K / RQ_BLOCK_CODES) * RQ_BLOCK_BYTES) return RQ_E_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(w_blocks_dev) & 255) != 0 || (reinterpret_cast<uintptr_t>(staging_dev) & 255) != 0) return RQ_E_WORKSPACE;
+    if (staging_bytes < inplace_staging_min(L)) return RQ_E_WORKSPACE;
+    if (gemm_fp6_enabled()) {
+        // wide batches read the fp6 plane: a weight without one cannot be served
+        if (!plane6_dev) return RQ_E_ARGUMENT;
+        if (plane6_bytes < L.bytes - L.off_w6 || (reinterpret_cast<uintptr_t>(plane6_dev) & 255) != 0) return RQ_E_WORKSPACE;
+    }
+    hipError_t e = init_rotate_quant_kernels();
+    if (e == hipSuccess) e = init_rotate_slab_kernels();
+    if (e == hipSuccess) e = init_decode_kernels();
+    if (e == hipSuccess) static_scratch(&e);
+    device_compute_units();
+    if (e != hipSuccess) return (int) e;
+    return (int) launch_prepare_inplace(w_blocks_dev, L, gemm_fp6_enabled() ? reinterpret_cast<uint8_t *>(plane6_dev) : nullptr,
+                                        reinterpret_cast<uint8_t *>(staging_dev), staging_bytes, (hipStream_t) stream);
+}
+
 size_t rq_w4a4_workspace_bytes(int type, int64_t K, int64_t N, int64_t M) {
     if (!shape_ok(type, K, N, M)) return 0;
     return workspace_layout(K, N, M < 1 ? 1 : M).bytes;

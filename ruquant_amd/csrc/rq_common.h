@@ -31,12 +31,15 @@ constexpr int kGemvMaxTokens = 64;  // workspaces of up to this many tokens hold
 //           an MFMA tile of 16 rows reads 256-byte runs.
 //   s_w   : n_panels x 64 floats (rows past N are zero).
 //   kmul  : n_panels x ng x 64 bytes, the integer weight multiplier of (row, group): 1 for legacy headers.
-//   flags : one int32; bit 0 set when any multiplier differs from 1 (kernels branch on it, uniformly).
+//   flags : one int32; bit 0 set when any multiplier differs from 1 (kernels branch on it, uniformly). At byte 8 of
+//           the section: the device address of the fp6 plane below (0: none), which the fp6 GEMM reads from there.
 //   w6    : (unless RQ_GEMM_FP6=0) the same codes once more as fp6 (E2M3) MFMA fragments for wide token batches:
 //           n_rtiles x ng x 8 fragments x 1536 bytes. Fragment f of row tile R (rows 256 R + 32 f ..), group g:
 //           lane l = row % 32 + 32 * half holds inputs 64 g + 32 half .. + 31 as 32 six-bit values (sign, then the
 //           magnitude 0 .. 8: as fp6 the value is code / 8), value j in bits 6j .. 6j+5 of the lane's 24 bytes; bytes
-//           0 .. 15 of lane l sit at l * 16, bytes 16 .. 23 at 1024 + l * 8. Rows past N are zero.
+//           0 .. 15 of lane l sit at l * 16, bytes 16 .. 23 at 1024 + l * 8. Rows past N are zero. A weight prepared in
+//           place (rq_w4a4_prepare_inplace) keeps the sections above in the tensor's own buffer and this plane in a
+//           buffer of its own.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kFrag6 = 1536;      // bytes of one 32 x 64 fp6 MFMA fragment
 constexpr int kRowTile6 = 256;    // rows of one tile of the fp6 plane
@@ -319,6 +322,17 @@ int device_compute_units();
 constexpr int kXcds = 8;
 
 hipError_t launch_prepare(const void *blocks, const PreparedLayout &L, uint8_t *prepared, hipStream_t stream);
+// in place: `blocks` becomes the prepared sections up to the flags (L.off_flags + 256 bytes, which must fit the
+// tensor), the fp6 plane goes to plane6 (may be null); staging: inplace_staging_min(L) bytes at the least
+hipError_t launch_prepare_inplace(void *blocks, const PreparedLayout &L, uint8_t *plane6, uint8_t *staging,
+                                  size_t staging_bytes, hipStream_t stream);
+inline size_t inplace_side_bytes(const PreparedLayout &L) {
+    return align_up((size_t) L.n_panels * kPanelRows * sizeof(float), 256) +
+           align_up((size_t) L.n_panels * L.ng * kPanelRows, 256) + 256;
+}
+inline size_t inplace_staging_min(const PreparedLayout &L) {
+    return inplace_side_bytes(L) + (size_t) kPanelRows * (L.ng / 4) * RQ_BLOCK_BYTES;
+}
 
 bool hadamard_factor(int64_t n, int &p, int &m);
 

@@ -403,7 +403,7 @@ __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, 
 
 template <int GS>
 __global__ void __launch_bounds__(kThreads)
-rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
+rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                 const int32_t *__restrict__ flags, const uint8_t *__restrict__ act6, const float *__restrict__ m4,
                 const float *__restrict__ u, float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng,
                 int n_panels, int n_tok_tiles, int n_tiles, int super_tiles, int n_whole, int parts,
@@ -455,6 +455,9 @@ rq_gemm6_kernel(const uint8_t *__restrict__ w6, const float *__restrict__ s_w, c
 #ifdef RQ6_STAMPS
     const long long ts0 = clock64();
 #endif
+    // the fp6 plane's address stands beside the flag word (it is inside the prepared buffer, or, for a weight that was
+    // prepared in place, a buffer of its own)
+    const uint8_t *w6 = reinterpret_cast<const uint8_t *>((uintptr_t) *reinterpret_cast<const unsigned long long *>(flags + 2));
     Ctx c;
     c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     c.wr = c.wave & 3;
@@ -698,7 +701,7 @@ hipError_t launch_gemm6(const GemmArgs &a, hipStream_t stream) {
     const int grid = pl.n_whole + (pl.n_tiles - pl.n_whole) * pl.parts;
     const float *m4 = reinterpret_cast<const float *>(a.act8 + act6_plane_bytes(a.L.ng, a.Mp));
 #define RQ_LAUNCH6(GS)                                                                                              \
-    hipLaunchKernelGGL(rq_gemm6_kernel<GS>, dim3(grid), dim3(kThreads), 0, stream, p + a.L.off_w6,                    \
+    hipLaunchKernelGGL(rq_gemm6_kernel<GS>, dim3(grid), dim3(kThreads), 0, stream,                                    \
                        reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,                           \
                        reinterpret_cast<const int32_t *>(p + a.L.off_flags), a.act8, m4, a.u, a.y, a.ldy, a.L.N, a.M, \
                        a.Mp, a.L.ng, a.L.n_panels, n_tok_tiles, pl.n_tiles, super_tiles, pl.n_whole, pl.parts,      \

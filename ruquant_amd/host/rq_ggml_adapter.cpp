@@ -10,8 +10,10 @@ namespace {
 struct rq_first_use {
     float   clip;
     int64_t n_rot;
-    void   *prepared;
+    void   *prepared;        // the tensor's own buffer (prepared in place) or a buffer of this struct's
     size_t  prepared_bytes;
+    void   *plane6;          // in place: the fp6 plane of the wide-batch kernel, which does not fit the tensor's buffer
+    bool    owns_prepared;
 };
 
 [[noreturn]] void rq_abort(const char *what, long long a = 0, long long b = 0) {
@@ -88,16 +90,43 @@ rq_first_use *first_use(rq_backend_context &ctx, const rq_tensor *src0) {
         rq_abort("W4A4H: Hadamard length does not divide this row slice (ruquant convert --rot-blocks)", hdr.pad[0],
                  src0->ne[0]);
     }
-    fu->prepared_bytes = rq_w4a4_prepared_bytes(src0->ne[0], src0->ne[1]);
-    hip_check(hipMalloc(&fu->prepared, fu->prepared_bytes), "prepared weight");
     if (rq_w4a4_weight_group(&hdr) == 64 && rq_w4a4_act_group() != 64) {
         // ggml_vec_dot_w4a4_a4 asserts the same (P:169-170): one weight multiplier per activation group
         rq_abort("weight groups of 64 need activation groups of 64 (RQ_ACT_GROUP)", rq_w4a4_act_group());
     }
-    const int rc = rq_w4a4_prepare(src0->data, src0->ne[0], src0->ne[1], fu->prepared, fu->prepared_bytes, ctx.stream);
-    if (rc != 0) rq_abort("rq_w4a4_prepare failed", rc);
-    // the workspace of every later call with up to max_tokens tokens: allocated now, outside capture
-    scratch(ctx, workspace_for(src0->type, src0->ne[0], src0->ne[1], ctx.max_tokens));
+    const int64_t K = src0->ne[0], N = src0->ne[1];
+    fu->prepared_bytes = rq_w4a4_prepared_bytes(K, N);
+    fu->plane6 = nullptr;
+    fu->owns_prepared = true;
+    // the workspace of every later call with up to max_tokens tokens: allocated now, outside capture; it also stages
+    // the in-place rewrite
+    size_t ws_bytes = workspace_for(src0->type, K, N, ctx.max_tokens);
+    const size_t staging = rq_w4a4_inplace_staging_bytes(K, N);
+    if (ctx.in_place && staging > ws_bytes) ws_bytes = staging;
+    void *ws = scratch(ctx, ws_bytes);
+    int rc = RQ_E_WORKSPACE;
+    if (ctx.in_place && (reinterpret_cast<uintptr_t>(src0->data) & 255) == 0) {
+        const size_t n6 = rq_w4a4_plane6_bytes(K, N);
+        if (n6) hip_check(hipMalloc(&fu->plane6, n6), "fp6 plane");
+        rc = rq_w4a4_prepare_inplace(src0->data, K, N, fu->plane6, n6, ws, ctx.scratch_bytes, ctx.stream);
+        if (rc == 0) {
+            fu->prepared = src0->data;
+            fu->owns_prepared = false;
+            // the staging area held blocks: the split-K cells inside the scratch must read zero again
+            hip_check(hipMemsetAsync(ctx.scratch, 0, ctx.scratch_bytes, stream), "scratch");
+            ctx.act.valid = false;
+        } else if (rc != RQ_E_WORKSPACE) {
+            rq_abort("rq_w4a4_prepare_inplace failed", rc);
+        } else if (fu->plane6) {   // (a shape whose prepared form does not fit its blocks: out of place after all)
+            hip_check(hipFree(fu->plane6), "fp6 plane");
+            fu->plane6 = nullptr;
+        }
+    }
+    if (rc != 0) {
+        hip_check(hipMalloc(&fu->prepared, fu->prepared_bytes), "prepared weight");
+        rc = rq_w4a4_prepare(src0->data, K, N, fu->prepared, fu->prepared_bytes, ctx.stream);
+        if (rc != 0) rq_abort("rq_w4a4_prepare failed", rc);
+    }
     const_cast<rq_tensor *>(src0)->extra = fu;
     return fu;
 }
@@ -205,7 +234,8 @@ void ggml_cuda_rq_graph_begin(rq_backend_context &ctx) { ctx.act.valid = false; 
 void ggml_cuda_rq_w4a4_release(rq_tensor *src0) {
     rq_first_use *fu = (rq_first_use *) src0->extra;
     if (!fu) return;
-    (void) hipFree(fu->prepared);
+    if (fu->owns_prepared) (void) hipFree(fu->prepared);
+    if (fu->plane6) (void) hipFree(fu->plane6);
     delete fu;
     src0->extra = nullptr;
 }

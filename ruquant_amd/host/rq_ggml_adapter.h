@@ -45,6 +45,10 @@ struct rq_backend_context {
     void        *scratch = nullptr;
     size_t       scratch_bytes = 0;
     int64_t      max_tokens = 512;
+    // first use rewrites a weight's own buffer into the prepared form, as the reference does (P:2046-2075): one copy of
+    // the codes stays resident and the tensor is no longer readable as blocks. false: the prepared form goes to a
+    // buffer of its own and the tensor's bytes stay valid ggml blocks (twice the memory).
+    bool         in_place = true;
     rq_act_cache act;
     long long    act_hits = 0, act_misses = 0;
     ~rq_backend_context();

@@ -102,6 +102,9 @@ int main(int argc, char **argv) {
     CK(hipStreamCreate(&stream));
     rq_backend_context ctx;
     ctx.stream = stream;
+    // RQ_HOST_IN_PLACE=0: keep the tensor's bytes as blocks and the prepared weight in a buffer of its own
+    const char *ip = getenv("RQ_HOST_IN_PLACE");
+    ctx.in_place = ip ? atoi(ip) != 0 : true;
 
     rq_tensor w = weight_tensor(type, K, N, wd), x = f32_tensor(K, M, xd), y = f32_tensor(N, M, yd);
     y.op = RQ_GGML_OP_MUL_MAT;
@@ -127,10 +130,21 @@ int main(int argc, char **argv) {
 
     const bool ready_before = ggml_cuda_rq_w4a4_ready(&w);
     bool fused_ran = false;
-    // first evaluation: first use of every weight, unfused (as the reference's graph gate forces)
+    // first evaluation: first use of every weight, unfused (as the reference's graph gate forces). Device memory taken
+    // by the first use of the LAST weight (the scratch buffer has its size by then when the weights have one shape) =
+    // what stays resident for a weight besides its tensor.
+    size_t free_before = 0, free_after = 0, total_mem = 0;
     ggml_cuda_rq_graph_begin(ctx);
-    ggml_cuda_mul_mat_rq_w4a4(ctx, &w, &x, &y);
     if (fuse) ggml_cuda_mul_mat_rq_w4a4(ctx, &w2, &x, &y2);
+    CK(hipStreamSynchronize(stream));
+    const size_t scratch_before = ctx.scratch_bytes;
+    CK(hipMemGetInfo(&free_before, &total_mem));
+    ggml_cuda_mul_mat_rq_w4a4(ctx, &w, &x, &y);
+    CK(hipStreamSynchronize(stream));
+    CK(hipMemGetInfo(&free_after, &total_mem));
+    const long long first_use_bytes = (long long) free_before - (long long) free_after -
+                                      ((long long) ctx.scratch_bytes - (long long) scratch_before);
+    if (fuse) ggml_cuda_mul_mat_rq_w4a4(ctx, &w2, &x, &y2);   // (in the order of the graph: after w)
     CK(hipStreamSynchronize(stream));
     const bool ready_after = ggml_cuda_rq_w4a4_ready(&w);
 
@@ -200,9 +214,13 @@ int main(int argc, char **argv) {
     }
     printf("{\"supported\": true, \"device\": \"%s\", \"type\": %d, \"K\": %lld, \"N\": %lld, \"M\": %lld, "
            "\"ready_before\": %s, \"ready_after\": %s, \"fused\": %s, \"iters\": %d, \"best_us\": %.2f, \"mean_us\": %.2f, "
-           "\"act_hits_first\": %lld, \"act_misses_first\": %lld, \"act_hits_again\": %lld, \"act_misses_again\": %lld}\n",
+           "\"act_hits_first\": %lld, \"act_misses_first\": %lld, \"act_hits_again\": %lld, \"act_misses_again\": %lld, "
+           "\"in_place\": %s, \"tensor_bytes\": %lld, \"first_use_bytes_beside_tensor\": %lld, \"plane6_bytes\": %lld, "
+           "\"prepared_bytes\": %lld}\n",
            prop.name, type, (long long) K, (long long) N, (long long) M, ready_before ? "true" : "false",
            ready_after ? "true" : "false", fused_ran ? "true" : "false", iters, iters ? best : 0.0,
-           iters ? sum / iters : 0.0, hits_first, misses_first, hits_again, misses_again);
+           iters ? sum / iters : 0.0, hits_first, misses_first, hits_again, misses_again, ctx.in_place ? "true" : "false",
+           (long long) w_bytes, first_use_bytes, (long long) rq_w4a4_plane6_bytes(K, N),
+           (long long) rq_w4a4_prepared_bytes(K, N));
     return 0;
 }

@@ -40,6 +40,10 @@ PROTOTYPES = {
     "rq_w4a4_prepared_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64]),
     "rq_w4a4_prepare": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
                                        ctypes.c_size_t, ctypes.c_void_p]),
+    "rq_w4a4_plane6_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64]),
+    "rq_w4a4_inplace_staging_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64]),
+    "rq_w4a4_prepare_inplace": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
+                                               ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "rq_w4a4_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64]),
     "rq_w4a4_mul_mat": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
                                        ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,

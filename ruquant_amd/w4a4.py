@@ -70,7 +70,7 @@ class W4A4Weight:
     """A W4A4 / W4A4H weight tensor on the GPU: [N, K/256] blocks as ggml stores them, plus what the first use
     derives (clip, Hadamard length, the prepared streaming form)."""
 
-    def __init__(self, blocks, type_, device="cuda:0", keep_blocks=True):
+    def __init__(self, blocks, type_, device="cuda:0", keep_blocks=True, in_place=False):
         blocks = np.ascontiguousarray(blocks)
         assert blocks.dtype == BLOCK_DTYPE and blocks.ndim == 2
         self.type = int(type_)
@@ -92,11 +92,26 @@ class W4A4Weight:
         nbytes = L.rq_w4a4_prepared_bytes(self.K, self.N)
         if nbytes == 0:
             raise RqError("unsupported weight shape K=%d N=%d" % (self.K, self.N))
-        self.prepared = _device_bytes(nbytes, self.device)
-        with torch.cuda.device(self.device):
-            _check(L.rq_w4a4_prepare(raw.data_ptr(), self.K, self.N, self.prepared.data_ptr(), nbytes,
-                                     _stream_ptr()), "rq_w4a4_prepare")
-        self.blocks = raw if keep_blocks else None
+        self.plane6 = None
+        if in_place:
+            # as the reference repacks (patch lines 2046-2075): the tensor's own buffer becomes the prepared weight
+            # (one copy of the codes resident), the fp6 plane of the wide-batch kernel lives beside it
+            n6 = L.rq_w4a4_plane6_bytes(self.K, self.N)
+            self.plane6 = _device_bytes(n6, self.device) if n6 else None
+            staging = _device_bytes(L.rq_w4a4_inplace_staging_bytes(self.K, self.N), self.device)
+            with torch.cuda.device(self.device):
+                _check(L.rq_w4a4_prepare_inplace(raw.data_ptr(), self.K, self.N,
+                                                 self.plane6.data_ptr() if n6 else None, n6, staging.data_ptr(),
+                                                 staging.numel(), _stream_ptr()), "rq_w4a4_prepare_inplace")
+                torch.cuda.current_stream().synchronize()   # staging is released below
+            self.prepared = raw
+            self.blocks = None
+        else:
+            self.prepared = _device_bytes(nbytes, self.device)
+            with torch.cuda.device(self.device):
+                _check(L.rq_w4a4_prepare(raw.data_ptr(), self.K, self.N, self.prepared.data_ptr(), nbytes,
+                                         _stream_ptr()), "rq_w4a4_prepare")
+            self.blocks = raw if keep_blocks else None
         self.ready = True
 
     def workspace(self, M):

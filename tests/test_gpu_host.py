@@ -21,12 +21,12 @@ def test_host_binary_is_built_and_prints_usage():
     assert r.returncode == 2 and "usage" in r.stderr
 
 
-def _run(tmp_path, type_, K, N, M, blocks, x, extra=()):
+def _run(tmp_path, type_, K, N, M, blocks, x, extra=(), env=None):
     blocks.tofile(tmp_path / "w.bin")
     x.tofile(tmp_path / "x.bin")
     cmd = [HOST, str(type_), str(K), str(N), str(M), str(tmp_path / "w.bin"), str(tmp_path / "x.bin"),
            str(tmp_path / "y.bin"), "3"] + [str(e) for e in extra]
-    r = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=120, env=env)
     return r, (np.fromfile(tmp_path / "y.bin", dtype=np.float32).reshape(M, N) if r.returncode == 0 else None)
 
 
@@ -150,3 +150,63 @@ def test_python_shared_activation_layer_chain(oracle):
         for n, r in (("o", ro), ("gate", rg), ("up", ru), ("down", rd)):
             got = out[n].cpu().numpy()
             assert bits_equal(got, r), "M=%d %s: %s" % (M, n, first_mismatch(got, r))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M", [1, 8, 200])
+def test_host_keeps_one_copy_of_the_codes(oracle, tmp_path, M):
+    """First use through the adapter rewrites the weight's own buffer (the reference's in-place repack, patch lines
+    2046-2075): beside the tensor only the fp6 plane of the wide-batch kernel stays resident, not a second copy of the
+    codes, and the results are the oracle's bits. With RQ_HOST_IN_PLACE=0 the prepared weight is a buffer of its own
+    (the tensor stays readable as blocks) and the same bits come out."""
+    type_, K, N = rq.TYPE_W4A4H, 5120, 4096
+    blocks = synth.random_weight_blocks(N, K, 41, type_, clip=0.9)
+    x = synth.activations("student_t4", M, K, 42)
+    want = oracle.mul_mat(type_, blocks, x, float(np.float32(0.9)), n_rot=K)
+    info = {}
+    for in_place in (1, 0):
+        env = dict(os.environ)
+        env["RQ_HOST_IN_PLACE"] = str(in_place)
+        # (a second weight of the same shape goes first, so that the scratch buffer has its size when the memory
+        # around the first use of the weight under test is read)
+        blocks.tofile(tmp_path / "w2.bin")
+        r, y = _run(tmp_path, type_, K, N, M, blocks, x, extra=("fuse", tmp_path / "w2.bin", N, tmp_path / "y2.bin"), env=env)
+        assert r.returncode == 0, r.stderr
+        info[in_place] = json.loads(r.stdout.strip().splitlines()[-1])
+        assert info[in_place]["in_place"] == bool(in_place)
+        assert bits_equal(y, want), "in_place=%d: %s" % (in_place, first_mismatch(y, want))
+    slack = 4 << 20                       # the allocator's granularity
+    a, b = info[1], info[0]
+    assert a["tensor_bytes"] == N * (K // 256) * 144
+    assert abs(a["first_use_bytes_beside_tensor"] - a["plane6_bytes"]) <= slack, a
+    assert abs(b["first_use_bytes_beside_tensor"] - b["prepared_bytes"]) <= slack, b
+    # in place: nothing of the size of the codes (N K / 2) is held twice
+    assert a["first_use_bytes_beside_tensor"] <= b["first_use_bytes_beside_tensor"] - N * K // 2 + slack
+
+
+@pytest.mark.gpu
+def test_prepare_in_place_python_binding(oracle):
+    """rq_w4a4_prepare_inplace through the Python binding over the token counts of every product kernel, ragged row
+    counts, weight multipliers and a long row; a shape too small to hold its prepared form in place is refused."""
+    import torch
+    dev = "cuda:0"
+    from tests.gpu_util import adversarial_weights, adversarial_activations, run_gpu
+    for type_, N, K, wgroup in ((rq.TYPE_W4A4H, 1000, 5120, 0), (rq.TYPE_W4A4, 777, 1024, 64),
+                                (rq.TYPE_W4A4H, 320, 17408, 256), (rq.TYPE_W4A4H, 4100, 256, 0)):
+        blocks, wf = adversarial_weights(oracle, N, K, type_, wgroup=wgroup)
+        W = rq.W4A4Weight(blocks, type_, dev, in_place=True)
+        assert W.blocks is None and W.prepared.numel() == blocks.nbytes
+        for M in (1, 3, 16, 70, 300):
+            x = adversarial_activations(M, K, type_, wf, seed=M)
+            got = run_gpu(W, x)
+            want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=max(W.n_rot, 0))
+            assert bits_equal(got, want), "N=%d K=%d M=%d: %s" % (N, K, M, first_mismatch(got, want))
+    L = rq.load_library()
+    tiny = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    stage = torch.zeros(L.rq_w4a4_inplace_staging_bytes(256, 3), dtype=torch.uint8, device=dev)
+    n6 = L.rq_w4a4_plane6_bytes(256, 3)
+    p6 = torch.zeros(max(n6, 256), dtype=torch.uint8, device=dev)
+    # three rows of one block each: 432 bytes of blocks cannot hold a panel of 64 padded rows
+    rc = L.rq_w4a4_prepare_inplace(tiny.data_ptr(), 256, 3, p6.data_ptr(), n6, stage.data_ptr(), stage.numel(), None)
+    assert rc == -2
+    torch.cuda.synchronize()
