@@ -125,22 +125,30 @@ struct Ctx {
     int wave, wr, wc, lane;
     int n_steps;             // steps (two groups each) of this workgroup
     int g0;                  // its first group
+#ifdef RQ6_STAMPS
+    long long ph[4];
+#endif
 };
 
-// fetch of the next step (two groups) into stage s, then advance the sources; past the last step they stay where they
-// are (the last step is fetched again, into cells nobody reads), so every step issues the same number of loads
-__device__ __forceinline__ void fetch(Ctx &c, Stage &s, int st) {
-    const uint32_t lane_off = (uint32_t) c.lane * 16;
-    const bool more = st + 1 < c.n_steps;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        load_run(c.run_src[i], lane_off, &s.cell[(i * 8 + c.wave) * 64]);
-        c.run_src[i] = uniform(c.run_src[i] + (more ? c.run_step[i] : 0));
-    }
+// fetch of step `st` (two groups) into stage s, then advance the sources; past the last step they stay where they
+// are (the last step is fetched again, into cells nobody reads), so every step issues the same number of loads.
+// In pieces, so that the loop can deal them out between its MFMAs: five loads issued back to back by all eight
+// wavefronts right behind the barrier queue up in front of the memory pipeline, and a wavefront that waits to issue a
+// load issues no MFMA either.
+__device__ __forceinline__ void fetch_run(Ctx &c, Stage &s, int st, int i) {
+    load_run(c.run_src[i], (uint32_t) c.lane * 16, &s.cell[(i * 8 + c.wave) * 64]);
+    c.run_src[i] = uniform(c.run_src[i] + (st + 1 < c.n_steps ? c.run_step[i] : 0));
+}
+__device__ __forceinline__ void fetch_tail(Ctx &c, Stage &s, int st) {
 #ifndef RQ6_NOTAIL
     load_cells(c.tail_src, &s.cell[kTailCell + c.wave * kTailLanes], ((uint64_t) 1 << kTailLanes) - 1);
 #endif
-    c.tail_src += more ? c.tail_step : 0;
+    c.tail_src += st + 1 < c.n_steps ? c.tail_step : 0;
+}
+__device__ __forceinline__ void fetch(Ctx &c, Stage &s, int st) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fetch_run(c, s, st, i);
+    fetch_tail(c, s, st);
 }
 
 __device__ __forceinline__ v8i fragment(const Stage &s, int cell0, int lane) {
@@ -314,15 +322,16 @@ __device__ __forceinline__ void read_operands(const Ctx &c, const Stage &s, int 
 
 // the four tiles of one group; the fold of a tile runs behind the MFMA of the next one, the last tile's result is
 // handed to the next group (P, pm, and the tile it belongs to is always (1, 1))
-template <bool HASK>
+template <bool HASK, class Between>
 __device__ __forceinline__ void group_units(const Ctx &c, const Operands &o, int g, v16f &P, float &pm,
-                                            float (&acc)[2][2][16], int32_t (&tot)[2][2][16]) {
+                                            float (&acc)[2][2][16], int32_t (&tot)[2][2][16], Between between) {
     const v16f zero = {};
 #pragma unroll
     for (int un = 0; un < 4; ++un) {
         const int a = un >> 1, b = un & 1;
         const int pa = un == 0 ? 1 : (un - 1) >> 1, pb = un == 0 ? 1 : (un - 1) & 1;
         const v16f S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.A[a], o.B[b], zero, 2, 2, 0, 0, 0, 0);
+        between(un);   // (a piece of the next stages' fetch: behind the MFMA, in front of the previous tile's fold)
         if (!HASK) {
             fold_fast(P, pm, acc[pa][pb]);
         } else {
@@ -355,10 +364,14 @@ __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, 
     }
     v16f P = {};
     float pm = 0.0f;
+    // stages 0 and 1 whole, of stage 2 the first three runs: its other two loads and everything after them is dealt
+    // out between the MFMAs of the loop (three runs of step st + 3 behind the barrier of step st, the fourth run and the
+    // fifth load in the first half of step st + 1)
     fetch(c, s0, 0);
     fetch(c, s1, 1);
-    fetch(c, s2, 2);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerStep) : "memory");
+#pragma unroll
+    for (int i = 0; i < 3; ++i) fetch_run(c, s2, 2, i);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerStep - 2) : "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     read_operands(c, s0, 0, X);
@@ -369,19 +382,42 @@ __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, 
             if (j > 0 && st >= c.n_steps) break;   // (wave-uniform)
             const Stage &cur = *ring[j];
             const Stage &next = *ring[(j + 1) % kRing];
-            Stage &refill = *ring[(j + 3) % kRing];
+            Stage &refill2 = *ring[(j + 2) % kRing];
+            Stage &refill3 = *ring[(j + 3) % kRing];
+#ifdef RQ6_STAMPS
+            const long long tp0 = __builtin_readcyclecounter();
+#endif
             if (RQ6_VARIANT != 3 && RQ6_VARIANT != 5) read_operands(c, cur, 1, Y);
             __builtin_amdgcn_sched_barrier(0);
-            group_units<HASK>(c, X, c.g0 + 2 * st, P, pm, acc, tot);
+            group_units<HASK>(c, X, c.g0 + 2 * st, P, pm, acc, tot, [&](int un) {
+                if (RQ6_VARIANT == 1 || RQ6_VARIANT == 5 || RQ6_VARIANT == 7) return;
+                if (un == 0) fetch_run(c, refill2, st + 2, 3);
+                if (un == 2) fetch_tail(c, refill2, st + 2);
+            });
+#ifdef RQ6_STAMPS
+            const long long tp1 = __builtin_readcyclecounter();
+#endif
             // stage st + 1 is whole once every wavefront has seen its own loads of it arrive (those of step st + 2
             // may still be in flight); stage st - 1 is then free for step st + 3
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerStep) : "memory");
+#ifdef RQ6_STAMPS
+            const long long tp2 = __builtin_readcyclecounter();
+#endif
             if (RQ6_VARIANT != 4 && RQ6_VARIANT != 5 && RQ6_VARIANT != 6) __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (RQ6_VARIANT != 1 && RQ6_VARIANT != 5 && RQ6_VARIANT != 7) fetch(c, refill, st + 3);
+#ifdef RQ6_STAMPS
+            const long long tp3 = __builtin_readcyclecounter();
+#endif
             if (RQ6_VARIANT != 3 && RQ6_VARIANT != 5) read_operands(c, next, 0, X);   // (past the last step: stale cells, never used)
             __builtin_amdgcn_sched_barrier(0);
-            group_units<HASK>(c, Y, c.g0 + 2 * st + 1, P, pm, acc, tot);
+            group_units<HASK>(c, Y, c.g0 + 2 * st + 1, P, pm, acc, tot, [&](int un) {
+                if (RQ6_VARIANT == 1 || RQ6_VARIANT == 5 || RQ6_VARIANT == 7) return;
+                if (un < 3) fetch_run(c, refill3, st + 3, un);
+            });
+#ifdef RQ6_STAMPS
+            const long long tp4 = __builtin_readcyclecounter();
+            c.ph[0] += tp1 - tp0; c.ph[1] += tp2 - tp1; c.ph[2] += tp3 - tp2; c.ph[3] += tp4 - tp3;
+#endif
         }
         if (!HASK && ((st0 / kRing + 1) % (kFlushSteps / kRing)) == 0) flush(acc, tot);
     }
@@ -465,6 +501,9 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
     c.lane = tid & 63;
     c.n_steps = s_end - s_begin;
     c.g0 = 2 * s_begin;
+#ifdef RQ6_STAMPS
+    c.ph[0] = c.ph[1] = c.ph[2] = c.ph[3] = 0;
+#endif
 #ifndef RQ6_SRC
 #define RQ6_SRC 0
 #endif
@@ -643,7 +682,8 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
         long long *dbg = reinterpret_cast<long long *>(y) + (size_t) blockIdx.x * 8;
         unsigned hwid = __builtin_amdgcn_s_getreg((32 - 1) << 11 | 0 << 6 | 4);
         unsigned xcc = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 0 << 6 | 20);
-        dbg[0] = ts0; dbg[1] = ts1; dbg[2] = ts2; dbg[3] = clock64(); dbg[4] = hwid; dbg[5] = xcc; dbg[6] = row_tile; dbg[7] = t0;
+        dbg[0] = ts0; dbg[1] = ts1; dbg[2] = ts2; dbg[3] = clock64(); dbg[4] = c.ph[0]; dbg[5] = c.ph[1]; dbg[6] = c.ph[2]; dbg[7] = c.ph[3];
+        (void) hwid; (void) xcc;
     }
 #endif
 }
