@@ -34,6 +34,9 @@
 
 #pragma clang fp contract(off)
 
+// Timing-only builds (-DRQ6_VARIANT=n, results are wrong): the loop with one ingredient left out, to see what each
+// costs. 1: no fetches; 2: no MFMAs or folds (groups of 128 / 256 only); 3: operands made up in registers instead of
+// read from LDS; 4: no barrier; 5: MFMAs and folds alone (1 + 3 + 4).
 #ifndef RQ6_VARIANT
 #define RQ6_VARIANT 0
 #endif
@@ -41,6 +44,11 @@
 namespace rq {
 
 namespace {
+
+constexpr bool kWithFetch = RQ6_VARIANT != 1 && RQ6_VARIANT != 5;
+constexpr bool kWithCompute = RQ6_VARIANT != 2;
+constexpr bool kWithLdsReads = RQ6_VARIANT != 3 && RQ6_VARIANT != 5;
+constexpr bool kWithBarrier = RQ6_VARIANT != 4 && RQ6_VARIANT != 5;
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -61,11 +69,7 @@ static_assert(kStageCells == 2368, "stage size");
 // cells) and 40 lanes' worth of a fifth (cells 2048 .. 2367: the rest of the activations and the multipliers).
 constexpr int kTailCell = 2048, kTailLanes = 40;
 static_assert(kTailCell + 8 * kTailLanes == kStageCells, "tail split");
-#ifndef RQ6_NOTAIL
 constexpr int kLoadsPerStep = 5;
-#else
-constexpr int kLoadsPerStep = 4;
-#endif
 
 constexpr int kXposeStride = 68;               // floats between tokens of a wavefront's output block in LDS (64 rows + 4)
 constexpr float kBias = 12582912.0f;           // 1.5 x 2^23
@@ -125,9 +129,6 @@ struct Ctx {
     int wave, wr, wc, lane;
     int n_steps;             // steps (two groups each) of this workgroup
     int g0;                  // its first group
-#ifdef RQ6_STAMPS
-    long long ph[4];
-#endif
 };
 
 // fetch of step `st` (two groups) into stage s, then advance the sources; past the last step they stay where they
@@ -140,9 +141,7 @@ __device__ __forceinline__ void fetch_run(Ctx &c, Stage &s, int st, int i) {
     c.run_src[i] = uniform(c.run_src[i] + (st + 1 < c.n_steps ? c.run_step[i] : 0));
 }
 __device__ __forceinline__ void fetch_tail(Ctx &c, Stage &s, int st) {
-#ifndef RQ6_NOTAIL
     load_cells(c.tail_src, &s.cell[kTailCell + c.wave * kTailLanes], ((uint64_t) 1 << kTailLanes) - 1);
-#endif
     c.tail_src += st + 1 < c.n_steps ? c.tail_step : 0;
 }
 __device__ __forceinline__ void fetch(Ctx &c, Stage &s, int st) {
@@ -256,14 +255,11 @@ template <bool HASK, int GS>
 __device__ __forceinline__ void step(Ctx &c, const Stage &cur, Stage &refill, int st, float (&acc)[2][2][16],
                                      int32_t (&tot)[2][2][16], v16f (&carry)[2][2]) {
     // the loads of steps st + 1 and st + 2 may still be in flight
-#ifndef RQ6_VARIANT
-#define RQ6_VARIANT 0
-#endif
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerStep) : "memory");
-    if (RQ6_VARIANT != 4 && RQ6_VARIANT != 5 && RQ6_VARIANT != 6) __builtin_amdgcn_s_barrier();
+    if (kWithBarrier) __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (RQ6_VARIANT != 1 && RQ6_VARIANT != 5 && RQ6_VARIANT != 7) fetch(c, refill, st + 3);
-    if (RQ6_VARIANT != 2) compute<HASK, GS>(c, cur, st, acc, tot, carry);
+    if (kWithFetch) fetch(c, refill, st + 3);
+    if (kWithCompute) compute<HASK, GS>(c, cur, st, acc, tot, carry);
 }
 
 __device__ __forceinline__ void flush(float (&acc)[2][2][16], int32_t (&tot)[2][2][16]) {
@@ -358,7 +354,7 @@ __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, 
                                        int32_t (&tot)[2][2][16]) {
     Stage *ring[kRing] = { &s0, &s1, &s2, &s3 };
     Operands X, Y;
-    if (RQ6_VARIANT == 3 || RQ6_VARIANT == 5) {
+    if (!kWithLdsReads) {
         for (int i = 0; i < 2; ++i) for (int e = 0; e < 6; ++e) { X.A[i][e] = c.lane * (e + 1); X.B[i][e] = c.lane * (e + i + 3); Y.A[i][e] = c.lane * (e + 7); Y.B[i][e] = c.lane * (e + i + 2); }
         X.m4[0] = X.m4[1] = Y.m4[0] = Y.m4[1] = 4.0f;
     }
@@ -384,40 +380,24 @@ __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, 
             const Stage &next = *ring[(j + 1) % kRing];
             Stage &refill2 = *ring[(j + 2) % kRing];
             Stage &refill3 = *ring[(j + 3) % kRing];
-#ifdef RQ6_STAMPS
-            const long long tp0 = __builtin_readcyclecounter();
-#endif
-            if (RQ6_VARIANT != 3 && RQ6_VARIANT != 5) read_operands(c, cur, 1, Y);
+            if (kWithLdsReads) read_operands(c, cur, 1, Y);
             __builtin_amdgcn_sched_barrier(0);
             group_units<HASK>(c, X, c.g0 + 2 * st, P, pm, acc, tot, [&](int un) {
-                if (RQ6_VARIANT == 1 || RQ6_VARIANT == 5 || RQ6_VARIANT == 7) return;
+                if (!kWithFetch) return;
                 if (un == 0) fetch_run(c, refill2, st + 2, 3);
                 if (un == 2) fetch_tail(c, refill2, st + 2);
             });
-#ifdef RQ6_STAMPS
-            const long long tp1 = __builtin_readcyclecounter();
-#endif
             // stage st + 1 is whole once every wavefront has seen its own loads of it arrive (those of step st + 2
             // may still be in flight); stage st - 1 is then free for step st + 3
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerStep) : "memory");
-#ifdef RQ6_STAMPS
-            const long long tp2 = __builtin_readcyclecounter();
-#endif
-            if (RQ6_VARIANT != 4 && RQ6_VARIANT != 5 && RQ6_VARIANT != 6) __builtin_amdgcn_s_barrier();
+            if (kWithBarrier) __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-#ifdef RQ6_STAMPS
-            const long long tp3 = __builtin_readcyclecounter();
-#endif
-            if (RQ6_VARIANT != 3 && RQ6_VARIANT != 5) read_operands(c, next, 0, X);   // (past the last step: stale cells, never used)
+            if (kWithLdsReads) read_operands(c, next, 0, X);   // (past the last step: stale cells, never used)
             __builtin_amdgcn_sched_barrier(0);
             group_units<HASK>(c, Y, c.g0 + 2 * st + 1, P, pm, acc, tot, [&](int un) {
-                if (RQ6_VARIANT == 1 || RQ6_VARIANT == 5 || RQ6_VARIANT == 7) return;
+                if (!kWithFetch) return;
                 if (un < 3) fetch_run(c, refill3, st + 3, un);
             });
-#ifdef RQ6_STAMPS
-            const long long tp4 = __builtin_readcyclecounter();
-            c.ph[0] += tp1 - tp0; c.ph[1] += tp2 - tp1; c.ph[2] += tp3 - tp2; c.ph[3] += tp4 - tp3;
-#endif
         }
         if (!HASK && ((st0 / kRing + 1) % (kFlushSteps / kRing)) == 0) flush(acc, tot);
     }
@@ -488,9 +468,6 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
     const int s_begin = sliced ? (int) ((int64_t) (ng / 2) * part / parts) : 0;
     const int s_end = sliced ? (int) ((int64_t) (ng / 2) * (part + 1) / parts) : ng / 2;
     const int tid = threadIdx.x;
-#ifdef RQ6_STAMPS
-    const long long ts0 = clock64();
-#endif
     // the fp6 plane's address stands beside the flag word (it is inside the prepared buffer, or, for a weight that was
     // prepared in place, a buffer of its own)
     const uint8_t *w6 = reinterpret_cast<const uint8_t *>((uintptr_t) *reinterpret_cast<const unsigned long long *>(flags + 2));
@@ -501,19 +478,9 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
     c.lane = tid & 63;
     c.n_steps = s_end - s_begin;
     c.g0 = 2 * s_begin;
-#ifdef RQ6_STAMPS
-    c.ph[0] = c.ph[1] = c.ph[2] = c.ph[3] = 0;
-#endif
-#ifndef RQ6_SRC
-#define RQ6_SRC 0
-#endif
-    const uint8_t *w_tile = w6 + (size_t) ((RQ6_SRC & 1) ? 0 : row_tile) * ng * (kCellsA * 16);   // this tile's rows, group 0
-#ifndef RQ6_BCONTIG
+    const uint8_t *w_tile = w6 + (size_t) row_tile * ng * (kCellsA * 16);   // this tile's rows, group 0
     const size_t a_step = (size_t) (Mp / 32) * kFrag6;                       // bytes between groups of the activation plane
-#else
-    const size_t a_step = (size_t) 4 * kFrag6;
-#endif
-    const uint8_t *a_tile = act6 + (size_t) (((RQ6_SRC & 2) ? 0 : t0) / 32) * kFrag6;              // this tile's tokens, group 0
+    const uint8_t *a_tile = act6 + (size_t) (t0 / 32) * kFrag6;              // this tile's tokens, group 0
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         // run L of the stage: runs 0 .. 23 are the weights of the step's two groups (12 each), 24 .. 35 the activations
@@ -565,9 +532,6 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
         }
     }
     const bool hask = flags[0] & 1;
-#ifdef RQ6_STAMPS
-    const long long ts1 = clock64();
-#endif
     // fp32 rounding toward minus infinity for the folds (MODE bits 1:0); the MFMA sums are exact in any mode
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2" ::: "memory");
     if (hask) {
@@ -578,9 +542,6 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
         else body<false, GS>(c, s0, s1, s2, s3, acc, tot);
         flush(acc, tot);
     }
-#ifdef RQ6_STAMPS
-    const long long ts2 = clock64();
-#endif
     // back to round to nearest even for the epilogue; the totals pass through the statement so that none of the
     // conversions below can be scheduled in front of it
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0" ::: "memory");
@@ -676,16 +637,6 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
             }
         }
     }
-#ifdef RQ6_STAMPS
-    __syncthreads();
-    if (tid == 0) {
-        long long *dbg = reinterpret_cast<long long *>(y) + (size_t) blockIdx.x * 8;
-        unsigned hwid = __builtin_amdgcn_s_getreg((32 - 1) << 11 | 0 << 6 | 4);
-        unsigned xcc = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 0 << 6 | 20);
-        dbg[0] = ts0; dbg[1] = ts1; dbg[2] = ts2; dbg[3] = clock64(); dbg[4] = c.ph[0]; dbg[5] = c.ph[1]; dbg[6] = c.ph[2]; dbg[7] = c.ph[3];
-        (void) hwid; (void) xcc;
-    }
-#endif
 }
 
 }  // namespace
