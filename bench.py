@@ -41,7 +41,7 @@ INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA
 HEADLINE_PROFILE = os.path.join(ROOT, "profiles", "decode_m1_k5120_n17408.md")
 
 
-GEMM_PROFILE = os.path.join(ROOT, "profiles", "gemm_m2048.md")   # "traffic_bytes_per_launch_m2048: <n>", both launches
+GEMM_PROFILE = os.path.join(ROOT, "profiles", "rq_gemm6_kernel_m2048_m512.md")   # "traffic_bytes_per_launch_m2048: <n>"
 
 
 def profiled_traffic_bytes(path=HEADLINE_PROFILE, key="traffic_bytes_per_launch:"):
