@@ -383,7 +383,7 @@ def machine_peaks(torch, rq, code_bytes, batches=5):
     t = mix(0)
     out["mfma_i8_16x16x64_tops_two_wavefronts_per_simd"] = round(cus * 8 * mi * 16 * ops_per_mfma / t / 1e6, 1)
     for op, name in ((0, "v_add_u32"), (1, "v_ashrrev_i32"), (2, "v_mul_i32_i24"), (3, "v_dot8c_i32_i4"),
-                     (4, "v_fma_f32")):
+                     (4, "v_fma_f32"), (5, "v_add_f32")):
         t1, t2 = mix(4, op), mix(1, op)
         out["valu_ns_per_instruction_per_simd_%s" % name] = {"one_wavefront": round(t1 * 1e3 / (vi * 128), 3),
                                                              "two_wavefronts": round(t2 * 1e3 / (2 * vi * 128), 3)}

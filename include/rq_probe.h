@@ -24,7 +24,7 @@ extern "C" {
  *                    Sub-kinds: 0 all wavefronts MFMA; 1 all VALU; 2 wavefronts 0..3 MFMA and 4..7 VALU (one of each
  *                    per SIMD); 3 wavefronts 0..3 MFMA, others idle; 4 wavefronts 4..7 VALU, others idle; 5 / 6 every
  *                    wavefront 1 MFMA + 8 / 16 VALU interleaved; 7 every wavefront its MFMAs, then its VALU work.
- *                    VALU instruction: 0 v_add_u32, 1 v_ashrrev_i32, 2 v_mul_i32_i24, 3 v_dot8c_i32_i4, 4 v_fma_f32.
+ *                    VALU instruction: 0 v_add_u32, 1 v_ashrrev_i32, 2 v_mul_i32_i24, 3 v_dot8c_i32_i4, 4 v_fma_f32, 5 v_add_f32.
  *                    MFMA form: 0 v_mfma_i32_16x16x64_i8 (with every VALU instruction), 1 v_mfma_i32_32x32x32_i8,
  *                    2 v_mfma_f32_32x32x64_f8f6f4 on fp8 operands, 3 the same on fp6 operands (forms 1..3 with VALU
  *                    instructions 0 and 4). The SIMD id each wavefront of workgroup 0 ran on is written to the 8 ints

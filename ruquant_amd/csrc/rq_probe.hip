@@ -62,6 +62,7 @@ __global__ void __launch_bounds__(256) probe_stream_kernel(const v4u *__restrict
         if (OPK == 2) RQ_VALU8("v_mul_i32_i24");          \
         if (OPK == 3) RQ_VALU8("v_dot8c_i32_i4");         \
         if (OPK == 4) RQ_FMA8();                          \
+        if (OPK == 5) RQ_VALU8("v_add_f32");              \
     } while (0)
 
 // Four independent accumulators of one MFMA form. MK: 0 v_mfma_i32_16x16x64_i8, 1 v_mfma_i32_32x32x32_i8,
@@ -107,7 +108,7 @@ struct Mfma<3> {
 //   SAME  = true : every wavefront interleaves 1 MFMA with NV VALU instructions (roles ignored)
 //   SAME  = false: wavefronts 0..3 take role_lo, wavefronts 4..7 role_hi
 // OPK: 0 = v_add_u32, 1 = v_ashrrev_i32, 2 = v_mul_i32_i24, 3 = v_dot8c_i32_i4, 4 = v_fma_f32 (eight chains of
-// dependent ones)
+// dependent ones), 5 = v_add_f32
 template <bool SAME, int NV, int OPK, int MK>
 __global__ void __launch_bounds__(512) probe_mix_kernel(int mfma_iters, int valu_iters, int role_lo, int role_hi,
                                                         int *sink, int *simd_of) {
@@ -239,6 +240,7 @@ extern "C" int rq_probe(int kind, int64_t a0, int64_t a1, int64_t a2, int64_t a3
                     case 2: RQ_MIX(2, 0);
                     case 3: RQ_MIX(3, 0);
                     case 4: RQ_MIX(4, 0);
+                    case 5: RQ_MIX(5, 0);
                     default: return RQ_E_ARGUMENT;
                 }
             }

@@ -23,7 +23,7 @@ def test_probe_kinds_launch_and_return():
         assert _probe(L, buf, STREAM, loads * 4096 * 16, loads, 0) == 0
     assert _probe(L, buf, STREAM, 1 << 22, 8, 64) == 0
     for sub in range(8):
-        for op in range(5):
+        for op in range(6):
             assert _probe(L, buf, MIX, sub | op << 8, 4, 2, 2) == 0
         for form in (1, 2, 3):   # the other MFMA forms, beside v_add_u32 and v_fma_f32
             for op in (0, 4):
@@ -45,7 +45,7 @@ def test_probe_argument_checks():
     assert _probe(L, buf, STREAM, 1 << 21, 8, 0) != 0          # more bytes than the buffer holds
     assert _probe(L, buf, STREAM, 12345, 8, 0) != 0            # not whole chunks
     assert _probe(L, buf, MIX, 8, 4, 2, 2) != 0                # unknown sub-kind
-    assert _probe(L, buf, MIX, 0 | 5 << 8, 4, 2, 2) != 0       # unknown VALU instruction
+    assert _probe(L, buf, MIX, 0 | 6 << 8, 4, 2, 2) != 0       # unknown VALU instruction
     assert _probe(L, buf, MIX, 0 | 2 << 8 | 3 << 20, 4, 2, 2) != 0   # a combination that is not built
     assert _probe(L, buf, MIX, 0, 0, 2, 2) != 0                # no workgroups
     assert _probe(L, buf, EMPTY, 256, nbytes=1024) != 0        # scratch too small
