@@ -50,6 +50,7 @@ constexpr bool kWithCompute = RQ6_VARIANT != 2;
 constexpr bool kWithLdsReads = RQ6_VARIANT != 3 && RQ6_VARIANT != 5;
 constexpr bool kWithBarrier = RQ6_VARIANT != 4 && RQ6_VARIANT != 5;
 
+typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) void lds_void;
@@ -75,6 +76,8 @@ constexpr int kXposeStride = 68;               // floats between tokens of a wav
 constexpr float kBias = 12582912.0f;           // 1.5 x 2^23
 constexpr int kBiasBits = 0x4B400000;
 constexpr int kFlushSteps = 16;                // 32 groups
+constexpr int kRsrcWord3 = 0x00020000;         // last word of a raw buffer descriptor on this target (32-bit data format)
+constexpr int kDeviceScope = 16;               // cache policy of a buffer access: the sc1 bit
 
 struct Stage {
     uint4 cell[kStageCells];
@@ -560,12 +563,19 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
         // workgroup counts the arrival. The workgroup that completes the count adds the other slices' slabs to the
         // totals it still holds and goes on to the epilogue; the others are done. (An atomic per output instead,
         // accumulating in 64-bit arrival cells, cost more than the slicing gained: 8 M device-scope atomics.)
-        unsigned long long *slab = slabs + ((size_t) slot * parts + part) * (kTileRows * kTileTok / 2);
+        // (Slabs move as 16 bytes per lane with the cache policy of a device-scope access: written through to memory,
+        // read past this XCD's L2.)
+        constexpr int kSlabBytes = kTileRows * kTileTok * (int) sizeof(int32_t);
+        uint8_t *slab_base = reinterpret_cast<uint8_t *>(slabs) + (size_t) slot * parts * kSlabBytes;
+        const uint32_t lane_off = (uint32_t) tid * 16;
+        {
+            const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(slab_base + (size_t) part * kSlabBytes, 0, kSlabBytes, kRsrcWord3);
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            const int a = i >> 4, b = (i >> 3) & 1, r = 2 * (i & 7);
-            const unsigned long long two = (unsigned long long) (uint32_t) tot[a][b][r] | (unsigned long long) (uint32_t) tot[a][b][r + 1] << 32;
-            __hip_atomic_store(slab + (size_t) i * kThreads + tid, two, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int i = 0; i < 16; ++i) {
+                const int a = i >> 3, b = (i >> 2) & 1, r = 4 * (i & 3);
+                __builtin_amdgcn_raw_buffer_store_b128(v4i{ tot[a][b][r], tot[a][b][r + 1], tot[a][b][r + 2], tot[a][b][r + 3] }, mine,
+                                                       lane_off + i * (kThreads * 16), 0, kDeviceScope);
+            }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's stores have reached memory
         __syncthreads();                                    // ... and everybody else's
@@ -577,15 +587,30 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
         }
         __syncthreads();
         if (*s_flag != parts - 1) return;
-        for (int pp = 0; pp < parts; ++pp) {
-            if (pp == part) continue;
-            const unsigned long long *other = slabs + ((size_t) slot * parts + pp) * (kTileRows * kTileTok / 2);
+        // the other parts' slabs, the loads of the next one in flight while one is added
+        v4i in[2][16];
+        auto load_part = [&](int k, v4i (&dst)[16]) {   // k-th of the other parts
+            const int pp = k < part ? k : k + 1;
+            const __amdgpu_buffer_rsrc_t other = __builtin_amdgcn_make_buffer_rsrc(slab_base + (size_t) pp * kSlabBytes, 0, kSlabBytes, kRsrcWord3);
 #pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                const int a = i >> 4, b = (i >> 3) & 1, r = 2 * (i & 7);
-                const unsigned long long two = __hip_atomic_load(other + (size_t) i * kThreads + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                tot[a][b][r] += (int32_t) (uint32_t) two;
-                tot[a][b][r + 1] += (int32_t) (uint32_t) (two >> 32);
+            for (int i = 0; i < 16; ++i) dst[i] = __builtin_amdgcn_raw_buffer_load_b128(other, lane_off + i * (kThreads * 16), 0, kDeviceScope);
+        };
+        auto add_part = [&](const v4i (&src)[16]) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int a = i >> 3, b = (i >> 2) & 1, r = 4 * (i & 3);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) tot[a][b][r + e] += src[i][e];
+            }
+        };
+        const int others = parts - 1;
+        load_part(0, in[0]);
+        for (int k = 0; k < others; k += 2) {
+            if (k + 1 < others) load_part(k + 1, in[1]);
+            add_part(in[0]);
+            if (k + 1 < others) {
+                if (k + 2 < others) load_part(k + 2, in[0]);
+                add_part(in[1]);
             }
         }
     }
