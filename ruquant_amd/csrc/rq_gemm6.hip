@@ -72,7 +72,7 @@ constexpr int kTailCell = 2048, kTailLanes = 40;
 static_assert(kTailCell + 8 * kTailLanes == kStageCells, "tail split");
 constexpr int kLoadsPerStep = 5;
 
-constexpr int kXposeStride = 68;               // floats between tokens of a wavefront's output block in LDS (64 rows + 4)
+constexpr int kXposeStride = 36;               // floats between tokens of a wavefront's output block in LDS (32 rows + 4)
 constexpr float kBias = 12582912.0f;           // 1.5 x 2^23
 constexpr int kBiasBits = 0x4B400000;
 constexpr int kFlushSteps = 16;                // 32 groups
@@ -429,7 +429,7 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                 int *__restrict__ counters, unsigned long long *__restrict__ slabs) {
     __shared__ Stage ring[kRing];
     Stage &s0 = ring[0], &s1 = ring[1], &s2 = ring[2], &s3 = ring[3];
-    static_assert(8 * 64 * kXposeStride * 4 <= sizeof(ring), "the epilogue's output blocks fit the ring");
+    static_assert(8 * 32 * kXposeStride * 4 <= sizeof(Stage), "the epilogue's output blocks fit one stage");
     // the epilogue's operands, fetched ahead of the first groups: the scales of the tile's 256 rows, then the units of
     // its 128 tokens
     __shared__ __align__(16) float s_pre[kTileRows + kTileTok + 4];   // (+ a word for the arrival count of a slice)
@@ -618,47 +618,47 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
     // epilogue (reference patch line 176): y = ((float(total) * 16) * u) * s_w. In the MFMA result a lane holds one
     // token (column) and, per tile, rows 8 q + 4 (lane / 32) + 0 .. 3 for q = 0 .. 3: stored as they are, a wavefront's
     // stores would be 32-byte pieces of 32 different rows of y (a third of the kernel's time went there). So every
-    // wavefront turns its 64 x 64 outputs through LDS (the ring is free now) and writes 256 contiguous bytes per token.
+    // wavefront turns its four 32 x 32 blocks through LDS one after the other (4.5 KiB per wavefront, all eight inside
+    // the last ring stage, which no fetch is aimed at when the loop ends) and writes 128 contiguous bytes per token.
     __syncthreads();   // every wavefront is done reading the ring
-    float *xp = reinterpret_cast<float *>(&s0.cell[0]) + c.wave * (64 * kXposeStride);   // s0 .. s3 are one 148 KiB block
+    float *xp = reinterpret_cast<float *>(&s3.cell[0]) + c.wave * (32 * kXposeStride);
     const int h = c.lane >> 5;
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-        const int tw = 32 * b + (c.lane & 31);   // token within the wavefront's 64
-        const float ut = s_pre[kTileRows + 64 * c.wc + tw];
+        const float ut = s_pre[kTileRows + 64 * c.wc + 32 * b + (c.lane & 31)];
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int rw = 32 * a + 8 * q + 4 * h;   // row within the wavefront's 64
-                const float4 sw = *reinterpret_cast<const float4 *>(&s_pre[64 * c.wr + rw]);
+                const int rw = 8 * q + 4 * h;   // row within the block
+                const float4 sw = *reinterpret_cast<const float4 *>(&s_pre[64 * c.wr + 32 * a + rw]);
                 float4 o;
                 o.x = (((float) tot[a][b][4 * q + 0] * 16.0f) * ut) * sw.x;
                 o.y = (((float) tot[a][b][4 * q + 1] * 16.0f) * ut) * sw.y;
                 o.z = (((float) tot[a][b][4 * q + 2] * 16.0f) * ut) * sw.z;
                 o.w = (((float) tot[a][b][4 * q + 3] * 16.0f) * ut) * sw.w;
-                *reinterpret_cast<float4 *>(&xp[tw * kXposeStride + rw]) = o;
+                *reinterpret_cast<float4 *>(&xp[(c.lane & 31) * kXposeStride + rw]) = o;
             }
-        }
-    }
-    // (a wavefront reads back only what it wrote itself: its LDS operations complete in order)
-    const int64_t n = (int64_t) row_tile * kTileRows + 64 * c.wr + 4 * (c.lane & 15);
+            // (a wavefront reads back only what it wrote itself, and its LDS operations complete in order)
+            const int64_t n = (int64_t) row_tile * kTileRows + 64 * c.wr + 32 * a + 4 * (c.lane & 7);
 #pragma unroll
-    for (int it = 0; it < 16; ++it) {
-        const int tw = 4 * it + (c.lane >> 4);
-        const int t = t0 + 64 * c.wc + tw;
-        const float4 o = *reinterpret_cast<const float4 *>(&xp[tw * kXposeStride + 4 * (c.lane & 15)]);
-        if (t >= M) continue;
-        float *dst = y + (int64_t) t * ldy + n;
-        if (n + 3 < N && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
-            // the output is written once and not read back by this launch: non-temporal
-            typedef float v4f __attribute__((ext_vector_type(4)));
-            __builtin_nontemporal_store(v4f{ o.x, o.y, o.z, o.w }, reinterpret_cast<v4f *>(dst));
-        } else {
-            const float ov[4] = { o.x, o.y, o.z, o.w };
+            for (int it = 0; it < 4; ++it) {
+                const int tw = 8 * it + (c.lane >> 3);   // token within the block
+                const int t = t0 + 64 * c.wc + 32 * b + tw;
+                const float4 o = *reinterpret_cast<const float4 *>(&xp[tw * kXposeStride + 4 * (c.lane & 7)]);
+                if (t >= M) continue;
+                float *dst = y + (int64_t) t * ldy + n;
+                if (n + 3 < N && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
+                    // the output is written once and not read back by this launch: non-temporal
+                    typedef float v4f __attribute__((ext_vector_type(4)));
+                    __builtin_nontemporal_store(v4f{ o.x, o.y, o.z, o.w }, reinterpret_cast<v4f *>(dst));
+                } else {
+                    const float ov[4] = { o.x, o.y, o.z, o.w };
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if (n + i < N) dst[i] = ov[i];
+                    for (int i = 0; i < 4; ++i) {
+                        if (n + i < N) dst[i] = ov[i];
+                    }
+                }
             }
         }
     }
