@@ -26,7 +26,7 @@ bad = W.clip != want_clip
 # the W4A4 variable is not set: a W4A4 tensor keeps clip 1
 W0 = rq.W4A4Weight(synth.random_weight_blocks(64, 256, 1, rq.TYPE_W4A4), rq.TYPE_W4A4, "cuda:0")
 bad |= W0.clip != 1.0
-for M in (1, 64, 512):
+for M in (1, 64, 512, 2048):   # (the last is benchmark configuration 3 at its full size: about a second of oracle)
     x = synth.activations("student_t4", M, K, 3)
     got = run_gpu(W, x)                                                      # the op takes W.clip, i.e. the environment's
     want = rq_oracle.mul_mat(rq.TYPE_W4A4H, blocks, x, want_clip, n_rot=K)
