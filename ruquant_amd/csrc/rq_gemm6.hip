@@ -329,7 +329,13 @@ __device__ __forceinline__ void group_units(const Ctx &c, const Operands &o, int
     for (int un = 0; un < 4; ++un) {
         const int a = un >> 1, b = un & 1;
         const int pa = un == 0 ? 1 : (un - 1) >> 1, pb = un == 0 ? 1 : (un - 1) & 1;
+        // The wavefront asks for issue priority while it hands over its MFMA. The two statements also pin the order
+        // MFMA, load, fold: without them the compiler moves the load (an assembly statement) in front of the MFMA,
+        // which then waits behind the load's issue (M=2048: 185.5 -> 180 us; with the priority left at 0 in both
+        // statements, 181 us).
+        __builtin_amdgcn_s_setprio(1);
         const v16f S = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(o.A[a], o.B[b], zero, 2, 2, 0, 0, 0, 0);
+        __builtin_amdgcn_s_setprio(0);
         between(un);   // (a piece of the next stages' fetch: behind the MFMA, in front of the previous tile's fold)
         if (!HASK) {
             fold_fast(P, pm, acc[pa][pb]);
