@@ -83,8 +83,11 @@ int rq_w4a4_weight_group(const void *host_block0);
 size_t rq_w4a4_prepared_bytes(int64_t K, int64_t N);
 
 /* Replaces rq_repack_once (P:2046-2075), out of place: reads N rows of K/256 blocks at w_blocks_dev, writes
- * prepared_dev (256-byte aligned, rq_w4a4_prepared_bytes). Asynchronous on `stream`; the input is not
- * modified and may be freed once the stream has passed this call. */
+ * prepared_dev (256-byte aligned, rq_w4a4_prepared_bytes). The input is not modified. Outside graph capture the
+ * call ends by waiting for `stream` and reading one word of the result back: whether the tensor carries weight
+ * multipliers, which the wide-batch launcher remembers per prepared address to choose between two kernels (both are
+ * right for every tensor; a prepared weight that is copied to another address, or prepared under capture, runs the
+ * one that is slow on tensors with multipliers). */
 int rq_w4a4_prepare(const void *w_blocks_dev, int64_t K, int64_t N,
                     void *prepared_dev, size_t prepared_bytes, rq_stream_t stream);
 

@@ -7,6 +7,7 @@
 #include <string.h>
 
 #include <mutex>
+#include <unordered_map>
 
 // Workspace of rq_w4a4_mul_mat_static: one array per GPU, part of the code object, so that callers which cannot
 // allocate device memory (HIP graph capture, serving loops) need none. In host code the array's name is only a handle
@@ -73,6 +74,41 @@ const Env &env() {
 }  // namespace
 
 bool gemm_fp6_enabled() { return env().gemm_fp6 != 0; }
+
+namespace {
+
+// Which prepared weights carry weight multipliers, for the weights this process has prepared: what the wide-batch
+// launcher chooses its kernel by. Only a hint: both kernels are right for every tensor (one is slow on tensors with
+// multipliers, the other a few percent slower on tensors without), so an address the table does not know, or knows
+// from a buffer that has since been reused, costs time at most.
+std::mutex g_notes_mutex;
+std::unordered_map<const void *, bool> g_notes;
+
+// reads the prepared weight's flag word back (first use synchronizes anyway); under graph capture nothing is noted
+void note_multipliers(const void *prepared, const PreparedLayout &L, hipStream_t stream) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    bool known = false, has = false;
+    if (hipStreamIsCapturing(stream, &st) == hipSuccess && st == hipStreamCaptureStatusNone) {
+        int32_t word = 0;
+        if (hipMemcpyAsync(&word, reinterpret_cast<const uint8_t *>(prepared) + L.off_flags, sizeof word, hipMemcpyDeviceToHost, stream) == hipSuccess &&
+            hipStreamSynchronize(stream) == hipSuccess) {
+            known = true;
+            has = (word & 1) != 0;
+        }
+    }
+    std::lock_guard<std::mutex> lock(g_notes_mutex);
+    if (known) g_notes[prepared] = has;
+    else g_notes.erase(prepared);
+}
+
+bool multipliers_noted(const void *prepared) {
+    std::lock_guard<std::mutex> lock(g_notes_mutex);
+    const auto it = g_notes.find(prepared);
+    return it != g_notes.end() && it->second;
+}
+
+}  // namespace
+
 
 namespace {
 
@@ -309,6 +345,7 @@ int run_products(int type, int n, const void *const *prepared, int64_t K, const 
             g.Mp = (int) W.Mp;
             g.groups_per_fold = G / kGroup;
             g.cells = have_slabs ? wsb + W.off_tot : nullptr;
+            g.weight_multipliers = multipliers_noted(fw.prepared[0]);
             e = fp6 ? launch_gemm6(g, stream) : launch_gemm(g, stream);
             if (e != hipSuccess) return (int) e;
         } else {
@@ -421,7 +458,9 @@ int rq_w4a4_prepare(const void *w_blocks_dev, int64_t K, int64_t N, void *prepar
     if (e == hipSuccess) static_scratch(&e);   // this device's address of the static workspace
     device_compute_units();
     if (e != hipSuccess) return (int) e;
-    return (int) launch_prepare(w_blocks_dev, L, reinterpret_cast<uint8_t *>(prepared_dev), (hipStream_t) stream);
+    e = launch_prepare(w_blocks_dev, L, reinterpret_cast<uint8_t *>(prepared_dev), (hipStream_t) stream);
+    if (e == hipSuccess) note_multipliers(prepared_dev, L, (hipStream_t) stream);
+    return (int) e;
 }
 
 size_t rq_w4a4_plane6_bytes(int64_t K, int64_t N) {
@@ -457,8 +496,10 @@ int rq_w4a4_prepare_inplace(void *w_blocks_dev, int64_t K, int64_t N, void *plan
     if (e == hipSuccess) static_scratch(&e);
     device_compute_units();
     if (e != hipSuccess) return (int) e;
-    return (int) launch_prepare_inplace(w_blocks_dev, L, gemm_fp6_enabled() ? reinterpret_cast<uint8_t *>(plane6_dev) : nullptr,
-                                        reinterpret_cast<uint8_t *>(staging_dev), staging_bytes, (hipStream_t) stream);
+    e = launch_prepare_inplace(w_blocks_dev, L, gemm_fp6_enabled() ? reinterpret_cast<uint8_t *>(plane6_dev) : nullptr,
+                               reinterpret_cast<uint8_t *>(staging_dev), staging_bytes, (hipStream_t) stream);
+    if (e == hipSuccess) note_multipliers(w_blocks_dev, L, (hipStream_t) stream);
+    return (int) e;
 }
 
 size_t rq_w4a4_workspace_bytes(int type, int64_t K, int64_t N, int64_t M) {

@@ -266,6 +266,7 @@ struct GemmArgs {
     int             M, Mp;
     int             groups_per_fold;   // 1; 2 or 4 when the activation groups are 128 or 256 wide
     void           *cells;             // fp6 form: arrival counters (zero on entry, left zero) and slabs of the tiles cut along K
+    bool            weight_multipliers = false;   // fp6 form: the host has seen this weight's flag for multipliers set
 };
 hipError_t launch_gemm(const GemmArgs &a, hipStream_t stream);
 // the fp6 form: act8 = the fp6 fragment plane with the multipliers behind it; the weight needs the fp6 plane

@@ -61,15 +61,18 @@ constexpr int kTileTok = 128;                  // tokens of a workgroup's tile
 constexpr int kCellsA = 8 * kFrag6 / 16;       // 768 cells: eight weight fragments of one group
 constexpr int kCellsB = 4 * kFrag6 / 16;       // 384 cells: four activation fragments of one group
 constexpr int kCellsM = kTileTok * 4 / 16;     // 32 cells: the 128 tokens' multipliers of one group (4 m as float)
-// One ring stage = two groups: [A g0][A g1][B g0][B g1][m g0][m g1] = 2368 cells of 16 bytes = 37 KiB
-constexpr int kOffA = 0, kOffB = 2 * kCellsA, kOffM = kOffB + 2 * kCellsB;
-constexpr int kStageCells = kOffM + 2 * kCellsM;
+// One ring stage = two groups: [A g0][A g1][B g0][B g1][m g0][m g1][k g0][k g1] = 2400 cells of 16 bytes = 37.5 KiB
+constexpr int kCellsK = kTileRows / 16;         // 16 cells: the 256 rows' weight multipliers of one group (a byte each)
+constexpr int kOffA = 0, kOffB = 2 * kCellsA, kOffM = kOffB + 2 * kCellsB, kOffK = kOffM + 2 * kCellsM;
+constexpr int kStageCellsPlain = kOffK;                 // without the rows' weight multipliers
+constexpr int kStageCellsK = kOffK + 2 * kCellsK;       // with them
 constexpr int kRing = 4;
-static_assert(kStageCells == 2368, "stage size");
+static_assert(kStageCellsPlain == 2368 && kStageCellsK == 2400, "stage size");
 // Each wavefront moves four whole 1 KiB runs per step (cells 0 .. 2047: the weights and the first 512 activation
-// cells) and 40 lanes' worth of a fifth (cells 2048 .. 2367: the rest of the activations and the multipliers).
-constexpr int kTailCell = 2048, kTailLanes = 40;
-static_assert(kTailCell + 8 * kTailLanes == kStageCells, "tail split");
+// cells) and 44 lanes' worth of a fifth (cells 2048 .. 2399: the rest of the activations, the tokens' multipliers and the
+// rows' weight multipliers).
+constexpr int kTailCell = 2048;
+static_assert(kTailCell + 8 * 40 == kStageCellsPlain && kTailCell + 8 * 44 == kStageCellsK, "tail split");
 constexpr int kLoadsPerStep = 5;
 
 constexpr int kXposeStride = 36;               // floats between tokens of a wavefront's output block in LDS (32 rows + 4)
@@ -79,8 +82,13 @@ constexpr int kFlushSteps = 16;                // 32 groups
 constexpr int kRsrcWord3 = 0x00020000;         // last word of a raw buffer descriptor on this target (32-bit data format)
 constexpr int kDeviceScope = 16;               // cache policy of a buffer access: the sc1 bit
 
-struct Stage {
-    uint4 cell[kStageCells];
+// WITHK: the stage of the kernel form that folds with weight multipliers from LDS. (Two layouts, because the 512
+// bytes shift the stages' LDS offsets, and with them the plain kernel's loop needs base registers it does not have.)
+template <bool WITHK>
+struct StageT {
+    static constexpr int kCells = WITHK ? kStageCellsK : kStageCellsPlain;
+    static constexpr int kTailLanes = WITHK ? 44 : 40;   // lanes of a wavefront's fifth load
+    uint4 cell[kCells];
 };
 
 // 64 lanes x 16 bytes from base + lane offset to 1 KiB of LDS at `lds` (wave-uniform; the hardware adds lane * 16).
@@ -127,7 +135,7 @@ struct Ctx {
     const uint8_t *run_src[4];
     size_t run_step[4];
     const uint8_t *tail_src; // this lane's cell of the fifth load, current step
-    size_t tail_step;        // its advance per step
+    uint32_t tail_step;      // its advance per step (bytes: under 4 GiB for any batch the workspace can hold)
     const uint8_t *k_src;    // weight multipliers of this wavefront's panel, row offset of the lane's first quad
     int wave, wr, wc, lane;
     int n_steps;             // steps (two groups each) of this workgroup
@@ -139,20 +147,24 @@ struct Ctx {
 // In pieces, so that the loop can deal them out between its MFMAs: five loads issued back to back by all eight
 // wavefronts right behind the barrier queue up in front of the memory pipeline, and a wavefront that waits to issue a
 // load issues no MFMA either.
+template <class Stage>
 __device__ __forceinline__ void fetch_run(Ctx &c, Stage &s, int st, int i) {
     load_run(c.run_src[i], (uint32_t) c.lane * 16, &s.cell[(i * 8 + c.wave) * 64]);
     c.run_src[i] = uniform(c.run_src[i] + (st + 1 < c.n_steps ? c.run_step[i] : 0));
 }
+template <class Stage>
 __device__ __forceinline__ void fetch_tail(Ctx &c, Stage &s, int st) {
-    load_cells(c.tail_src, &s.cell[kTailCell + c.wave * kTailLanes], ((uint64_t) 1 << kTailLanes) - 1);
+    load_cells(c.tail_src, &s.cell[kTailCell + c.wave * Stage::kTailLanes], ((uint64_t) 1 << Stage::kTailLanes) - 1);
     c.tail_src += st + 1 < c.n_steps ? c.tail_step : 0;
 }
+template <class Stage>
 __device__ __forceinline__ void fetch(Ctx &c, Stage &s, int st) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) fetch_run(c, s, st, i);
     fetch_tail(c, s, st);
 }
 
+template <class Stage>
 __device__ __forceinline__ v8i fragment(const Stage &s, int cell0, int lane) {
     const uint4 p0 = s.cell[cell0 + lane];
     const uint2 p1 = *(reinterpret_cast<const uint2 *>(&s.cell[cell0 + 64]) + lane);
@@ -169,7 +181,25 @@ __device__ __forceinline__ void fold_fast(const v16f &S, float m4, float (&acc)[
     for (int r = 0; r < 16; ++r) acc[r] = __builtin_fmaf(S[r], m4, acc[r]);
 }
 
-// weight multipliers: tot += floor(k m S / 16) in integers (reference patch line 173)
+// weight multipliers (reference patch lines 169-173): acc += floor(k m S / 16), the same single FMA with 4 m k in
+// place of 4 m (k <= 15, so a group moves the accumulator by at most 15 x 122,400: flush after every second group).
+// kw: the multipliers of the lane's sixteen rows, four bytes per register.
+__device__ __forceinline__ void fold_km(const v16f &S, float m4, const uint32_t (&kw)[4], float (&acc)[16]) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const float kf = (float) ((kw[r >> 2] >> (8 * (r & 3))) & 0xFFu);
+        acc[r] = __builtin_fmaf(S[r], kf * m4, acc[r]);
+    }
+}
+// the sixteen multipliers a lane needs for row block a (rows 32 a + 8 q + 4 (lane / 32) + 0 .. 3, q = 0 .. 3) of group gi
+template <class Stage>
+__device__ __forceinline__ void read_kw(const Ctx &c, const Stage &s, int gi, int a, uint32_t (&kw)[4]) {
+    const uint32_t *k = reinterpret_cast<const uint32_t *>(&s.cell[kOffK + gi * kCellsK]) + 16 * c.wr + 8 * a + (c.lane >> 5);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) kw[q] = k[2 * q];
+}
+
+// the same in integers, from multipliers in global memory (the forms for activation groups of 128 / 256)
 __device__ __forceinline__ void fold_k(const v16f &S, float m4, const int (&kk)[16], int32_t (&tot)[16]) {
     const int mi = (int) (m4 * 0.25f);
 #pragma unroll
@@ -182,7 +212,7 @@ __device__ __forceinline__ void fold_k(const v16f &S, float m4, const int (&kk)[
 // One step (two groups of 64 inputs) of one wavefront: 64 rows x 64 tokens as 2 x 2 tiles. GS = runs of 64 per
 // activation group (1, 2, 4). A unit = one tile x one activation group's runs inside this step: its MFMAs chain through
 // the accumulator operand; the fold of unit i runs behind the MFMAs of unit i + 1.
-template <bool HASK, int GS>
+template <bool HASK, int GS, class Stage>
 __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, int st, float (&acc)[2][2][16],
                                         int32_t (&tot)[2][2][16], v16f (&carry)[2][2]) {
     constexpr int kRuns = GS == 1 ? 1 : 2;        // runs of a unit inside one step
@@ -254,7 +284,7 @@ __device__ __forceinline__ void compute(const Ctx &c, const Stage &s, int st, fl
     }
 }
 
-template <bool HASK, int GS>
+template <bool HASK, int GS, class Stage>
 __device__ __forceinline__ void step(Ctx &c, const Stage &cur, Stage &refill, int st, float (&acc)[2][2][16],
                                      int32_t (&tot)[2][2][16], v16f (&carry)[2][2]) {
     // the loads of steps st + 1 and st + 2 may still be in flight
@@ -279,7 +309,7 @@ __device__ __forceinline__ void flush(float (&acc)[2][2][16], int32_t (&tot)[2][
     }
 }
 
-template <bool HASK, int GS>
+template <bool HASK, int GS, class Stage>
 __device__ __forceinline__ void body(Ctx &c, Stage &s0, Stage &s1, Stage &s2, Stage &s3,
                                      float (&acc)[2][2][16], int32_t (&tot)[2][2][16]) {
     v16f carry[2][2] = {};
@@ -310,6 +340,7 @@ struct Operands {
     float m4[2];
 };
 
+template <class Stage>
 __device__ __forceinline__ void read_operands(const Ctx &c, const Stage &s, int gi, Operands &o) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -321,14 +352,21 @@ __device__ __forceinline__ void read_operands(const Ctx &c, const Stage &s, int 
 
 // the four tiles of one group; the fold of a tile runs behind the MFMA of the next one, the last tile's result is
 // handed to the next group (P, pm, and the tile it belongs to is always (1, 1))
-template <bool HASK, class Between>
-__device__ __forceinline__ void group_units(const Ctx &c, const Operands &o, int g, v16f &P, float &pm,
-                                            float (&acc)[2][2][16], int32_t (&tot)[2][2][16], Between between) {
+// (with weight multipliers: `sk`, `gi` = the stage and the group in it that `o` was read from, `sp`, `gp` = those of
+// the group before it, whose last tile is folded behind this group's first MFMA; the multipliers of a fold's rows are
+// read from LDS in front of the MFMA that the fold stands behind)
+// KFMA: the one-FMA fold with multipliers from LDS; otherwise (a kernel that is launched when nothing says the tensor
+// has weight multipliers, and must still be right when it has) the integer fold with multipliers from global memory.
+template <bool HASK, bool KFMA, class Stage, class Between>
+__device__ __forceinline__ void group_units(const Ctx &c, const Operands &o, int g, const Stage &sp, int gp, const Stage &sk, int gi,
+                                            v16f &P, float &pm, float (&acc)[2][2][16], int32_t (&tot)[2][2][16], Between between) {
     const v16f zero = {};
 #pragma unroll
     for (int un = 0; un < 4; ++un) {
         const int a = un >> 1, b = un & 1;
         const int pa = un == 0 ? 1 : (un - 1) >> 1, pb = un == 0 ? 1 : (un - 1) & 1;
+        uint32_t kw[4];
+        if (HASK && KFMA) read_kw(c, un == 0 ? sp : sk, un == 0 ? gp : gi, pa, kw);
         // The wavefront asks for issue priority while it hands over its MFMA. The two statements also pin the order
         // MFMA, load, fold: without them the compiler moves the load (an assembly statement) in front of the MFMA,
         // which then waits behind the load's issue (M=2048: 185.5 -> 180 us; with the priority left at 0 in both
@@ -339,8 +377,10 @@ __device__ __forceinline__ void group_units(const Ctx &c, const Operands &o, int
         between(un);   // (a piece of the next stages' fetch: behind the MFMA, in front of the previous tile's fold)
         if (!HASK) {
             fold_fast(P, pm, acc[pa][pb]);
+        } else if (KFMA) {
+            fold_km(P, pm, kw, acc[pa][pb]);   // (a workgroup's first fold adds nothing: P and pm start as zero)
         } else {
-            const int pg = un == 0 ? g - 1 : g;   // (a workgroup's first fold adds nothing: P and pm start as zero)
+            const int pg = un == 0 ? g - 1 : g;
             int k16[16];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -358,7 +398,7 @@ __device__ __forceinline__ void group_units(const Ctx &c, const Operands &o, int
     }
 }
 
-template <bool HASK>
+template <bool HASK, bool KFMA, class Stage>
 __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, Stage &s3, float (&acc)[2][2][16],
                                        int32_t (&tot)[2][2][16]) {
     Stage *ring[kRing] = { &s0, &s1, &s2, &s3 };
@@ -391,7 +431,7 @@ __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, 
             Stage &refill3 = *ring[(j + 3) % kRing];
             if (kWithLdsReads) read_operands(c, cur, 1, Y);
             __builtin_amdgcn_sched_barrier(0);
-            group_units<HASK>(c, X, c.g0 + 2 * st, P, pm, acc, tot, [&](int un) {
+            group_units<HASK, KFMA>(c, X, c.g0 + 2 * st, *ring[(j + 3) % kRing], 1, cur, 0, P, pm, acc, tot, [&](int un) {
                 if (!kWithFetch) return;
                 if (un == 0) fetch_run(c, refill2, st + 2, 3);
                 if (un == 2) fetch_tail(c, refill2, st + 2);
@@ -403,16 +443,21 @@ __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, 
             asm volatile("" ::: "memory");
             if (kWithLdsReads) read_operands(c, next, 0, X);   // (past the last step: stale cells, never used)
             __builtin_amdgcn_sched_barrier(0);
-            group_units<HASK>(c, Y, c.g0 + 2 * st + 1, P, pm, acc, tot, [&](int un) {
+            group_units<HASK, KFMA>(c, Y, c.g0 + 2 * st + 1, cur, 0, cur, 1, P, pm, acc, tot, [&](int un) {
                 if (!kWithFetch) return;
                 if (un < 3) fetch_run(c, refill3, st + 3, un);
             });
+            if (HASK && KFMA) flush(acc, tot);   // (every accumulator has taken two groups' terms since the last one)
         }
         if (!HASK && ((st0 / kRing + 1) % (kFlushSteps / kRing)) == 0) flush(acc, tot);
     }
     // the last tile of the last group
     if (!HASK) {
         fold_fast(P, pm, acc[1][1]);
+    } else if (KFMA) {
+        uint32_t kw[4];
+        read_kw(c, *ring[(c.n_steps - 1) % kRing], 1, 1, kw);
+        fold_km(P, pm, kw, acc[1][1]);
     } else {
         int k16[16];
 #pragma unroll
@@ -426,13 +471,15 @@ __device__ __forceinline__ void body64(Ctx &c, Stage &s0, Stage &s1, Stage &s2, 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the refetches of the last steps
 }
 
-template <int GS>
+// KFMA (activation groups of 64 only): the form of the kernel for tensors with weight multipliers; see group_units
+template <int GS, bool KFMA>
 __global__ void __launch_bounds__(kThreads)
 rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
                 const int32_t *__restrict__ flags, const uint8_t *__restrict__ act6, const float *__restrict__ m4,
                 const float *__restrict__ u, float *__restrict__ y, int64_t ldy, int64_t N, int M, int Mp, int ng,
                 int n_panels, int n_tok_tiles, int n_tiles, int super_tiles, int n_whole, int parts,
                 int *__restrict__ counters, unsigned long long *__restrict__ slabs) {
+    using Stage = StageT<KFMA>;
     __shared__ Stage ring[kRing];
     Stage &s0 = ring[0], &s1 = ring[1], &s2 = ring[2], &s3 = ring[3];
     static_assert(8 * 32 * kXposeStride * 4 <= sizeof(Stage), "the epilogue's output blocks fit one stage");
@@ -505,15 +552,21 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
     }
     {
         // fifth load: cells 2048 .. 2303 are the last 256 cells of the second group's activations, cells 2304 .. 2367
-        // the multipliers of the two groups
-        const int cell = kTailCell + c.wave * kTailLanes + (c.lane < kTailLanes ? c.lane : 0);
+        // the tokens' multipliers of the two groups, cells 2368 .. 2399 the weight multipliers of the tile's 256 rows
+        // for the two groups (a byte per row: 64 bytes per panel of 64 rows)
+        const int cell = kTailCell + c.wave * Stage::kTailLanes + (c.lane < Stage::kTailLanes ? c.lane : 0);
         if (cell < kOffM) {
-            c.tail_step = 2 * a_step;
-            c.tail_src = a_tile + a_step + (size_t) (cell - (kOffB + kCellsB)) * 16 + s_begin * c.tail_step;
-        } else {
+            c.tail_step = (uint32_t) (2 * a_step);
+            c.tail_src = a_tile + a_step + (size_t) (cell - (kOffB + kCellsB)) * 16 + (size_t) s_begin * c.tail_step;
+        } else if (cell < kOffK) {
             const int gi = (cell - kOffM) / kCellsM, off = (cell - kOffM) % kCellsM;
-            c.tail_step = (size_t) 2 * Mp * sizeof(float);
-            c.tail_src = reinterpret_cast<const uint8_t *>(m4 + (size_t) gi * Mp + t0) + (size_t) off * 16 + s_begin * c.tail_step;
+            c.tail_step = (uint32_t) (2 * Mp * sizeof(float));
+            c.tail_src = reinterpret_cast<const uint8_t *>(m4 + (size_t) gi * Mp + t0) + (size_t) off * 16 + (size_t) s_begin * c.tail_step;
+        } else {
+            const int gi = (cell - kOffK) / kCellsK, x = (cell - kOffK) % kCellsK;
+            const int pnl = min(row_tile * 4 + (x >> 2), n_panels - 1);
+            c.tail_step = 2 * kPanelRows;
+            c.tail_src = kmul + ((size_t) pnl * ng + gi) * kPanelRows + (size_t) (x & 3) * 16 + (size_t) s_begin * c.tail_step;
         }
     }
     const int panel = min(row_tile * 4 + c.wr, n_panels - 1);
@@ -544,13 +597,13 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
     // fp32 rounding toward minus infinity for the folds (MODE bits 1:0); the MFMA sums are exact in any mode
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2" ::: "memory");
     if (hask) {
-        if constexpr (GS == 1) body64<true>(c, s0, s1, s2, s3, acc, tot);
+        if constexpr (GS == 1) body64<true, KFMA>(c, s0, s1, s2, s3, acc, tot);
         else body<true, GS>(c, s0, s1, s2, s3, acc, tot);
     } else {
-        if constexpr (GS == 1) body64<false>(c, s0, s1, s2, s3, acc, tot);
+        if constexpr (GS == 1) body64<false, KFMA>(c, s0, s1, s2, s3, acc, tot);
         else body<false, GS>(c, s0, s1, s2, s3, acc, tot);
-        flush(acc, tot);
     }
+    flush(acc, tot);
     // back to round to nearest even for the epilogue; the totals pass through the statement so that none of the
     // conversions below can be scheduled in front of it
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0" ::: "memory");
@@ -722,16 +775,19 @@ hipError_t launch_gemm6(const GemmArgs &a, hipStream_t stream) {
     const int super_tiles = n_tok_tiles % 4 == 0 && n_row_tiles % 8 == 0;
     const int grid = pl.n_whole + (pl.n_tiles - pl.n_whole) * pl.parts;
     const float *m4 = reinterpret_cast<const float *>(a.act8 + act6_plane_bytes(a.L.ng, a.Mp));
-#define RQ_LAUNCH6(GS)                                                                                              \
-    hipLaunchKernelGGL(rq_gemm6_kernel<GS>, dim3(grid), dim3(kThreads), 0, stream,                                    \
+#define RQ_LAUNCH6(GS, KFMA)                                                                                        \
+    hipLaunchKernelGGL((rq_gemm6_kernel<GS, KFMA>), dim3(grid), dim3(kThreads), 0, stream,                            \
                        reinterpret_cast<const float *>(p + a.L.off_sw), p + a.L.off_kmul,                           \
                        reinterpret_cast<const int32_t *>(p + a.L.off_flags), a.act8, m4, a.u, a.y, a.ldy, a.L.N, a.M, \
                        a.Mp, a.L.ng, a.L.n_panels, n_tok_tiles, pl.n_tiles, super_tiles, pl.n_whole, pl.parts,      \
                        reinterpret_cast<int *>(a.cells),                                                             \
                        reinterpret_cast<unsigned long long *>(reinterpret_cast<uint8_t *>(a.cells) + kGemm6CounterBytes))
-    if (a.groups_per_fold == 1) RQ_LAUNCH6(1);
-    else if (a.groups_per_fold == 2) RQ_LAUNCH6(2);
-    else RQ_LAUNCH6(4);
+    // (a.weight_multipliers: what the host knows about the tensor; only a choice between two kernels that are both
+    // right for every tensor)
+    if (a.groups_per_fold == 1 && a.weight_multipliers) RQ_LAUNCH6(1, true);
+    else if (a.groups_per_fold == 1) RQ_LAUNCH6(1, false);
+    else if (a.groups_per_fold == 2) RQ_LAUNCH6(2, false);
+    else RQ_LAUNCH6(4, false);
 #undef RQ_LAUNCH6
     return hipGetLastError();
 }

@@ -74,6 +74,63 @@ def test_slices_longest_row_extreme_sums(oracle):
     assert got[0, 0] == np.float32(expect)
 
 
+@pytest.mark.parametrize("per", [256, 64])
+def test_weight_multipliers_extreme_sums(oracle, per):
+    """The same extremes on a tensor with weight multipliers (rq.pack_groups, one per block or per 64 inputs): rows of
+    all -8 / all +7 codes with multiplier 15 everywhere against q - z = +-15 with m = 255. A group then moves the
+    biased accumulator by 15 x 122400 = 1.836 M, so the kernel for such tensors transfers it to the int32 total after
+    every second group (3.67 M of the 4.19 M of its window); whole tiles and K slices, both signs."""
+    N, K, M, type_ = 300, 4352, 1200, rq.TYPE_W4A4
+    rng = np.random.default_rng(17)
+    codes = rng.integers(-8, 8, size=(N, K), dtype=np.int8)
+    codes[0, :] = -8
+    codes[1, :] = 7
+    codes[2, :] = np.where((np.arange(K) // 64) % 2 == 0, -8, 7)
+    units = np.abs(rng.normal(0.02, 0.005, size=N)).astype(np.float32)
+    mults = rng.integers(1, 16, size=(N, K // per), dtype=np.int32)
+    mults[0:3, :] = 15
+    mults[5, :] = 1
+    blocks = rq.pack_groups(codes, units, mults)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    x = synth.activations("outlier_channels", M, K, 9)
+    x[0, :] = 1.0
+    x[1, :] = -1.0
+    x[2, :] = np.where((np.arange(K) // 64) % 2 == 0, 1.0, -1.0)
+    got = run_gpu(W, x)
+    sample = [0, 1, 2, 3, 127, 128, 640, 1199]
+    want = oracle.mul_mat(type_, blocks, x[sample], W.clip, n_rot=0)
+    assert bits_equal(got[sample], want), first_mismatch(got[sample], want)
+    unit = np.float32(1.0) / np.float32(3825.0)
+    expect = (np.float32(-15 * 122400 * (K // 64)) * np.float32(16.0)) * unit * units[0]
+    assert got[0, 0] == np.float32(expect)
+
+
+def test_weight_multipliers_at_an_address_the_library_has_not_seen(oracle):
+    """The launcher picks the kernel for tensors with weight multipliers from what rq_w4a4_prepare saw. A copy of the
+    prepared bytes at another address is unknown to it and takes the other kernel, which must give the same bits."""
+    import ctypes
+    import torch
+    N, K, M, type_ = 520, 2560, 200, rq.TYPE_W4A4H
+    blocks, wf = adversarial_weights(oracle, N, K, type_, wgroup=64)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    x_np = adversarial_activations(M, K, type_, wf)
+    want = oracle.mul_mat(type_, blocks, x_np, W.clip, n_rot=K)
+    assert bits_equal(run_gpu(W, x_np), want)
+    L = rq.load_library()
+    moved = torch.empty(W.prepared.numel() + 4096, dtype=torch.uint8, device=DEV)[2048:2048 + W.prepared.numel()]
+    assert moved.data_ptr() % 256 == 0
+    moved.copy_(W.prepared)
+    x = torch.from_numpy(x_np).to(DEV)
+    y = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+    ws = W.workspace(M)
+    rc = L.rq_w4a4_mul_mat(type_, moved.data_ptr(), K, N, x.data_ptr(), K, M, y.data_ptr(), N, W.clip, K, ws.data_ptr(),
+                           ws.numel(), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    got = y.cpu().numpy()
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
 @pytest.mark.parametrize("M", [65, 128, 129, 300])
 def test_token_counts_around_the_tile(oracle, M):
     """One and a few token tiles, partly filled, K = 5120 (every tile cut along K: few tiles, long rows)."""
