@@ -194,7 +194,12 @@ __device__ __forceinline__ void fold_km(const v16f &S, float m4, const uint32_t 
 // the sixteen multipliers a lane needs for row block a (rows 32 a + 8 q + 4 (lane / 32) + 0 .. 3, q = 0 .. 3) of group gi
 template <class Stage>
 __device__ __forceinline__ void read_kw(const Ctx &c, const Stage &s, int gi, int a, uint32_t (&kw)[4]) {
-    const uint32_t *k = reinterpret_cast<const uint32_t *>(&s.cell[kOffK + gi * kCellsK]) + 16 * c.wr + 8 * a + (c.lane >> 5);
+    // (the lane's part of the address is worked out here each time: kept across the loop, the eight addresses that the
+    // compiler forms from it, one per stage and group, are registers the loop does not have, and their reloads from
+    // scratch wait for every load in flight)
+    uint32_t h = (uint32_t) c.lane >> 5;
+    asm volatile("" : "+v"(h));
+    const uint32_t *k = reinterpret_cast<const uint32_t *>(&s.cell[kOffK + gi * kCellsK]) + 16 * c.wr + 8 * a + h;
 #pragma unroll
     for (int q = 0; q < 4; ++q) kw[q] = k[2 * q];
 }
@@ -596,7 +601,7 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
     const bool hask = flags[0] & 1;
     // fp32 rounding toward minus infinity for the folds (MODE bits 1:0); the MFMA sums are exact in any mode
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 2" ::: "memory");
-    if (hask) {
+    if (KFMA || hask) {   // (the form for weight multipliers takes every tensor that way: multipliers of 1 where there are none)
         if constexpr (GS == 1) body64<true, KFMA>(c, s0, s1, s2, s3, acc, tot);
         else body<true, GS>(c, s0, s1, s2, s3, acc, tot);
     } else {
@@ -604,8 +609,18 @@ rq_gemm6_kernel(const float *__restrict__ s_w, const uint8_t *__restrict__ kmul,
         else body<false, GS>(c, s0, s1, s2, s3, acc, tot);
     }
     flush(acc, tot);
-    // back to round to nearest even for the epilogue; the totals pass through the statement so that none of the
-    // conversions below can be scheduled in front of it
+    // Back to round to nearest even for the epilogue. The compiler does not know that fp32 arithmetic reads MODE, so
+    // the totals pass through a statement on either side of the change: the one in front keeps the last folds (which
+    // the totals depend on) from being scheduled behind it, the one behind keeps the conversions below from being
+    // scheduled in front of it.
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) asm volatile("" : "+v"(tot[a][b][r]));
+        }
+    }
     asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0" ::: "memory");
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
