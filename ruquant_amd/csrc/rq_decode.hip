@@ -65,8 +65,13 @@ struct DecodeKernelArgs {
     int          main_panels;       // whole panels per workgroup: panels s, s + G, ... (G = workgroups)
     int          tail_panel0;       // first panel of the remainder, which is dealt in quads of rows
     int          q_base, q_extra;   // remainder quads per workgroup: q_base, the first q_extra slots one more
-    int          n_pass;            // Sylvester passes through LDS after the register pass
     int          inv_nblk;          // floor(2^22 / nblk) + 1, nblk = K / 256: i / nblk = (i * inv_nblk) >> 22 for every item index
+    int          syncs;             // bits 0-7: times the rotate wavefronts meet (rot_sync) until the codes are in LDS
+                                    // bits 8-9: 1 / 2: every rotate wavefront has that many pairs of Paley items and
+                                    // quantizes their sums from its registers (paley_quantize); 0: the sums go through
+                                    // LDS. (One word: the arguments end where a 64-byte line of the kernel-argument
+                                    // segment ends, and a word on the next line is a miss that the first wait of
+                                    // every wavefront sits out: 1.2 us.)
 };
 
 __device__ __forceinline__ int dot8(uint32_t a, uint32_t b, int c) {
@@ -228,6 +233,181 @@ __device__ __forceinline__ void paley_pair(const float *buf, float *alt, int s, 
     }
 }
 
+// Maxima over the lanes of up to sixteen registers at once, each result delivered to the lanes that will work with
+// it: a butterfly in which a lane keeps one register of a pair and hands the other to its partner, so every level
+// halves the registers (three instructions per pair: two selects and a maximum whose operand is the lane permutation)
+// where one all-lanes reduction per register costs six plus a transfer through a scalar register. The partners are the
+// four exact lane exchanges of the DPP unit, in an order in which no exchange disturbs the lane bits chosen by earlier
+// levels: lane ^ 7 (row_half_mirror, choosing by lane bit 2), ^ 1 (bit 0), ^ 2 (bit 1), ^ 8 (row_ror:8, bit 3); then
+// the four rows of sixteen lanes are combined so that every row holds the results. Register i's result ends in the
+// lanes l with scatter_index(l) == i; lanes whose index has no register hold the identity.
+// SIGNED: maximum of the bit patterns as signed integers, which among floats of both signs is the largest positive
+// value if there is one (else some negative value: the caller takes the maximum with 0 anyway); otherwise as unsigned
+// integers: the most negative value if there is one.
+__device__ __forceinline__ int scatter_index(int lane) {
+    return ((lane >> 2) & 1) | ((lane & 1) << 1) | (((lane >> 1) & 1) << 2) | (lane & 8);
+}
+constexpr int scatter_lane(int i) { return ((i & 1) << 2) | ((i >> 1) & 1) | (((i >> 2) & 1) << 1) | (i & 8); }
+
+template <bool SIGNED>
+__device__ __forceinline__ uint32_t pattern_max(uint32_t a, uint32_t b) {
+    return SIGNED ? (uint32_t) max((int) a, (int) b) : max(a, b);
+}
+template <bool SIGNED, int LEVEL>
+__device__ __forceinline__ uint32_t exchange_max(uint32_t keep, uint32_t give) {
+    constexpr int kCtrl = LEVEL == 0 ? 0x141 : LEVEL == 1 ? 0xB1 : LEVEL == 2 ? 0x4E : 0x128;
+    return pattern_max<SIGNED>(keep, (uint32_t) __builtin_amdgcn_update_dpp(0, (int) give, kCtrl, 0xF, 0xF, true));
+}
+template <bool SIGNED, int N, int LEVEL>
+__device__ __forceinline__ uint32_t scatter_max(const uint32_t (&v)[N], const bool (&upper)[4]) {
+    constexpr uint32_t kIdentity = SIGNED ? 0x80000000u : 0u;
+    if constexpr (LEVEL == 4) {
+        static_assert(N == 1, "sixteen registers at most");
+        typedef unsigned v2u __attribute__((ext_vector_type(2)));
+        const v2u a = __builtin_amdgcn_permlane16_swap(v[0], v[0], false, false);   // rows 0 with 1, 2 with 3
+        const uint32_t r = pattern_max<SIGNED>(a.x, a.y);
+        const v2u b = __builtin_amdgcn_permlane32_swap(r, r, false, false);         // the halves of the wavefront
+        return pattern_max<SIGNED>(b.x, b.y);
+    } else {
+        constexpr int H = (N + 1) / 2;
+        uint32_t r[H];
+#pragma unroll
+        for (int j = 0; j < H; ++j) {
+            const uint32_t A = v[2 * j], B = 2 * j + 1 < N ? v[2 * j + 1] : kIdentity;
+            r[j] = exchange_max<SIGNED, LEVEL>(upper[LEVEL] ? B : A, upper[LEVEL] ? A : B);
+        }
+        return scatter_max<SIGNED, H, LEVEL + 1>(r, upper);
+    }
+}
+
+// Paley stage and activation quantizer of one rotate wavefront without a trip through LDS in between, for rows where
+// every wavefront has NPAIR pairs of Paley items (column runs cr, cr + 1, ... of slice s). The 64 lanes of one Paley
+// output register hold 64 neighbouring columns of one output chunk: exactly one activation group. So the group's
+// range is a reduction over the lanes of that register (reference lines 2646-2654), the lanes the reduction delivers
+// group i to work out its multiplier, zero point and reciprocal step (lines 2662-2668: the two divisions once per
+// group), and the codes are made where the values are (lines 2670-2675), eight neighbouring lanes gathering a code word.
+template <int P, int NPAIR>
+__device__ __forceinline__ void paley_quantize(const float *buf, int s, int cr, int lane, int wave, int lm, int m,
+                                               int n_rot, int pm, float scale, float clip, float *s_part,
+                                               float *s_unit, uint32_t *s_act, int32_t *s_mz, int *s_cnt,
+                                               int &sync_target, unsigned long long *stamps) {
+    (void) stamps;
+    constexpr int kOut = P / 4;
+    constexpr int NG = NPAIR * 2 * kOut;   // groups (= registers) of this wavefront
+    constexpr int NB = (NG + 15) / 16;     // batches of sixteen registers: batch b is delivered to the lanes of row b
+    static_assert(NB <= 2, "two rows of lanes take the parameters");
+    float x[NG];
+    int e0[NPAIR][2];   // element index of output 0 of the run's first column
+#pragma unroll
+    for (int pr = 0; pr < NPAIR; ++pr) {
+        const int c0 = (cr + 2 * pr) * 64 + lane, c1 = c0 + 64;
+        const int b0 = (c0 >> lm) * n_rot + (c0 & (m - 1)), b1 = (c1 >> lm) * n_rot + (c1 & (m - 1));
+        float out0[kOut], out1[kOut];
+        if (m == 256) {
+            paley_pick_stream2<P, kOut, 272>(s, buf + padi(b0), buf + padi(b1), 272, out0, out1);
+        } else {
+            paley_pick_stream2<P, kOut, 0>(s, buf + padi(b0), buf + padi(b1), pm, out0, out1);
+        }
+#pragma unroll
+        for (int o = 0; o < kOut; ++o) {
+            x[(2 * pr) * kOut + o] = out0[o] * scale;
+            x[(2 * pr + 1) * kOut + o] = out1[o] * scale;
+        }
+        e0[pr][0] = __builtin_amdgcn_readfirstlane(b0 + kOut * s * m);
+        e0[pr][1] = __builtin_amdgcn_readfirstlane(b1 + kOut * s * m);
+    }
+    RQ_STAMP_AT(stamps, 9);
+    RQ_STAMP_AT(stamps, 4);
+    RQ_STAMP_AT(stamps, 10);
+    // ranges: min(0, x ...) and max(0, x ...) of each register over its lanes, delivered to the lanes of the group
+    const bool upper[4] = { (lane & 4) != 0, (lane & 1) != 0, (lane & 2) != 0, (lane & 8) != 0 };
+    const int g_l = ((lane >> 4) & 1) * 16 + scatter_index(lane);   // the group (of this wavefront) the lane works for
+    uint32_t lo_bits = 0, hi_bits = 0;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        constexpr int kFull = 16;
+        const int n = NG - b * kFull < kFull ? NG - b * kFull : kFull;
+        uint32_t v[kFull];
+#pragma unroll
+        for (int i = 0; i < kFull; ++i) v[i] = b * kFull + i < NG ? __builtin_bit_cast(uint32_t, x[b * kFull + i < NG ? b * kFull + i : 0]) : 0u;
+        uint32_t lo_b, hi_b;
+        if (n > 8) {
+            lo_b = scatter_max<false, 16, 0>(v, upper);
+#pragma unroll
+            for (int i = 0; i < kFull; ++i) if (b * kFull + i >= NG) v[i] = 0x80000000u;
+            hi_b = scatter_max<true, 16, 0>(v, upper);
+        } else {
+            uint32_t w8[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) w8[i] = v[i];
+            lo_b = scatter_max<false, 8, 0>(w8, upper);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) if (b * kFull + i >= NG) w8[i] = 0x80000000u;
+            hi_b = scatter_max<true, 8, 0>(w8, upper);
+        }
+        if (b == 0 || (lane & 16)) {
+            lo_bits = lo_b;
+            hi_bits = hi_b;
+        }
+    }
+    const bool mine = g_l < NG && lane < 32;
+    const float lo_l = fminf(__builtin_bit_cast(float, lo_bits), 0.0f) * clip;
+    const float hi_l = fmaxf(__builtin_bit_cast(float, hi_bits), 0.0f) * clip;
+    const float rmax = wave_max(mine ? hi_l - lo_l : 0.0f);
+    if (lane == 0) s_part[wave] = rmax;
+    RQ_STAMP_AT(stamps, 11);
+    rot_sync(s_cnt, sync_target, lane);
+    RQ_STAMP_AT(stamps, 5);
+
+    float Rg = s_part[0];
+#pragma unroll
+    for (int i = 1; i < kRotWaves; ++i) Rg = fmaxf(Rg, s_part[i]);
+    if (Rg == 0.0f) Rg = 2.0f;
+    const float u = Rg / 3825.0f;  // 15 * 255
+    if (wave == 0 && lane == 0) s_unit[0] = u;
+    // the parameters of the lane's group
+    const int mg_l = (int) fminf(fmaxf(ceilf(((hi_l - lo_l) * 255.0f) / Rg), 1.0f), 255.0f);
+    const float inv_l = 1.0f / ((float) mg_l * u);
+    const float zf_l = fminf(fmaxf(rintf(-lo_l * inv_l), 0.0f), 15.0f);
+    if (mine) {
+        // (group g: run g / kOut of the wavefront, output g % kOut)
+        const int run = g_l / kOut, o = g_l - run * kOut;
+        int e = e0[0][0];
+#pragma unroll
+        for (int pr = 0; pr < NPAIR; ++pr) {
+            if (run == 2 * pr) e = e0[pr][0];
+            if (run == 2 * pr + 1) e = e0[pr][1];
+        }
+        s_mz[(e + o * m) >> 6] = mg_l | ((8 - (int) zf_l) & 0xFF) << 8;
+    }
+    // (all code words first, then the stores under one lane mask: with a store per group in between, every group's
+    // dependent chain ran alone, with the wait states of its lane permutations unfilled)
+    const int nib_shift = 4 * (lane & 7);
+    uint32_t word[NG];
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+        const int src = (i >> 4) * 16 + scatter_lane(i & 15);
+        const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, inv_l), src));
+        const float zf = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zf_l), src));
+        // (the median of three is the clamp: the sum is finite)
+        const uint32_t q = (uint32_t) (int) __builtin_amdgcn_fmed3f(rintf(x[i] * inv) + zf, 0.0f, 15.0f);
+        uint32_t w = q << nib_shift;
+        w |= (uint32_t) __builtin_amdgcn_update_dpp(0, (int) w, 0xB1, 0xF, 0xF, true);
+        w |= (uint32_t) __builtin_amdgcn_update_dpp(0, (int) w, 0x4E, 0xF, 0xF, true);
+        w |= (uint32_t) __builtin_amdgcn_update_dpp(0, (int) w, 0x141, 0xF, 0xF, true);
+        word[i] = w ^ 0x88888888u;   // q - 8 as 4-bit two's complement
+    }
+    if ((lane & 7) == 0) {
+        uint32_t *dst = s_act + (lane >> 3);
+#pragma unroll
+        for (int i = 0; i < NG; ++i) {
+            const int e = e0[i / (2 * kOut)][(i / kOut) & 1] + (i % kOut) * m;
+            dst[e >> 3] = word[i];
+        }
+    }
+    RQ_STAMP_AT(stamps, 12);
+}
+
 // MG: group-items (64 rows x one group: two loads) a stream wavefront has in flight per round of a whole panel;
 // MT: remainder items (8 rows x 4 groups: one load) per round. The first round of both is issued up front.
 template <int P, int MG, int MT>
@@ -370,7 +550,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
 
         const bool anyk = ((f0 | f1 | f2) & 1) != 0;
         const int n_items = n_oct * nblk;
-        const int codes_ready = kRotWaves * (1 + a.n_pass + (a.rotate ? 1 : 0) + 2);
+        const int codes_ready = kRotWaves * (a.syncs & 255);
         bool waited = false;
 
         // remainder item `i` of this workgroup -> address of its 1 KiB (8 rows x 4 groups x 2 halves)
@@ -542,6 +722,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
     } else {
         // =========================================================== the activation side (512 threads)
         const int rt = tid;
+        const int paley_pairs = a.syncs >> 8;
         int sync_target = 0;
         // the row (requested at the top of the kernel)
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -605,7 +786,21 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
                 const int col_runs = (ncols + 63) >> 6;
                 const int n_it = kSlices * col_runs;
                 const int per_wave = (n_it + kRotWaves - 1) / kRotWaves;
-                if (per_wave == 2 && (col_runs & 1) == 0 && (ncols & 63) == 0 && 2 * wave + 1 < n_it) {
+                if (paley_pairs) {
+                    // every wavefront has whole pairs of items: Paley sums, ranges and codes without leaving registers
+                    int s = 0, cr = per_wave * wave;
+                    while (cr >= col_runs) {
+                        cr -= col_runs;
+                        ++s;
+                    }
+                    if (paley_pairs == 1) {
+                        paley_quantize<P, 1>(buf, s, cr, lane, wave, lm, m, a.n_rot, pm, a.scale, a.clip, s_part, s_unit,
+                                             s_act, s_mz, s_cnt, sync_target, RQ_STAMP_PTR);
+                    } else {
+                        paley_quantize<P, 2>(buf, s, cr, lane, wave, lm, m, a.n_rot, pm, a.scale, a.clip, s_part, s_unit,
+                                             s_act, s_mz, s_cnt, sync_target, RQ_STAMP_PTR);
+                    }
+                } else if (per_wave == 2 && (col_runs & 1) == 0 && (ncols & 63) == 0 && 2 * wave + 1 < n_it) {
                     // the wavefront's two items are neighbouring column runs of one slice: one instruction stream
                     // for both (whole row rotated as H20 x H256 or H12 x H256: 16 items for eight wavefronts)
                     int s = 0, cr = 2 * wave;
@@ -651,18 +846,20 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
 #pragma unroll
                     for (int o = 0; o < kOut; ++o) dst[o * m] = out[o] * a.scale;
                 }
-                RQ_STAMP(9);
-                rot_sync(s_cnt, sync_target, lane);
+                if (!paley_pairs) {
+                    RQ_STAMP(9);
+                    rot_sync(s_cnt, sync_target, lane);
+                }
             } else {
                 for (int i = rt; i < K; i += kRotThreads) buf[padi(i)] = buf[padi(i)] * a.scale;
                 rot_sync(s_cnt, sync_target, lane);
             }
         }
 
-        RQ_STAMP(4);
         // ---- group ranges, the token's unit, multipliers, zero points and codes (quantize_rounds), with the number
         // of code words per thread as a compile-time constant
-        {
+        if (!(P > 1 && a.rotate && paley_pairs)) {
+            RQ_STAMP(4);
             const int nw = K >> 3;
             const bool dense = a.rotate && P > 1;            // the Paley stage wrote the dense buffer
             const float *row = dense ? alt : buf;
@@ -772,7 +969,20 @@ hipError_t launch_decode(const DecodeArgs &d, hipStream_t stream) {
     // stages through LDS: those above stride 8, or above stride 128 when the chunks are whole blocks of 256 floats
     // (four more stages then run between lanes)
     const int lm0 = d.rotate && (d.m & 255) == 0 ? 8 : 4;
-    k.n_pass = d.rotate && lm > lm0 ? (lm - lm0 + 3) / 4 : 0;
+    const int n_pass = d.rotate && lm > lm0 ? (lm - lm0 + 3) / 4 : 0;   // Sylvester passes through LDS after the register pass
+    int paley_pairs = 0;
+    if (d.rotate && d.p > 1 && d.K % d.p == 0) {
+        // the Paley items (4 slices x runs of 64 columns) deal out as one or two whole pairs of neighbouring runs to
+        // each of the eight rotate wavefronts: H20 x H256, H12 x H256 (one pair), H12 x H512, H20 x H512 (two)
+        const int ncols = d.K / d.p, col_runs = ncols / 64, n_it = 4 * col_runs;
+        const int per_wave = n_it / kRotWaves;
+        if ((ncols & 63) == 0 && (d.m & 63) == 0 && n_it == per_wave * kRotWaves && (per_wave == 2 || per_wave == 4) &&
+            col_runs % per_wave == 0) {
+            paley_pairs = per_wave / 2;
+        }
+    }
+    // meetings: row in LDS, the Sylvester passes, Paley (or the scale) unless the sums stay in registers, ranges, codes
+    k.syncs = (1 + n_pass + (d.rotate && !paley_pairs ? 1 : 0) + 2) | paley_pairs << 8;
     const int n_panels = k.ws.first[kMaxFused];
     // one workgroup per compute unit: whole panels as far as they go round, the remainder in quads of rows. More
     // workgroups (a multiple of the compute units) only when the rows of one would not fit its LDS cells.

@@ -416,6 +416,40 @@ def test_one_token_whole_panels(oracle, type_, K, N, n_rot, mult):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
+@pytest.mark.parametrize("K,n_rot", [(5120, 5120), (6144, 6144), (10240, 10240), (3072, 3072), (5120, 2560), (12288, 12288)])
+@pytest.mark.parametrize("row", ["zeros", "one_spike", "constant", "negative_constant", "signed_zeros", "alternating",
+                                 "one_group_only", "tiny"])
+def test_one_token_rows_that_press_the_group_ranges(oracle, K, n_rot, row):
+    """One token whose rotated row has groups without a negative value, without a positive one, all zero, or a range
+    far below the token's widest: the one-launch kernel reduces a group's range over the lanes of the register that
+    holds the group (bit patterns compared as integers, an identity for absent registers) and must land on the
+    reference's min / max chain from 0 (reference patch lines 2646-2654) in every such case. A constant row rotates
+    into a single non-zero value per Sylvester chunk; a spike rotates into a row of equal magnitudes."""
+    N, type_ = 192, rq.TYPE_W4A4H
+    blocks = synth.random_weight_blocks(N, K, 21, type_, clip=1.0, n_rot=n_rot)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    x = np.zeros((1, K), np.float32)
+    if row == "one_spike":
+        x[0, 77] = 3.0
+    elif row == "constant":
+        x[0, :] = 0.25
+    elif row == "negative_constant":
+        x[0, :] = -1.5
+    elif row == "signed_zeros":
+        x[0, ::2] = -0.0
+        x[0, 5] = 1.0
+        x[0, 6] = -1.0
+    elif row == "alternating":
+        x[0, :] = np.where(np.arange(K) % 2 == 0, 1.0, -1.0)
+    elif row == "one_group_only":
+        x[0, :] = synth.activations("outlier_channels", 1, K, 5)[0] * (np.arange(K) // 64 == 3)
+    elif row == "tiny":
+        x[0, :] = synth.activations("outlier_channels", 1, K, 6)[0] * np.float32(1e-30)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=n_rot)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
 @pytest.mark.parametrize("M", [1, 12, 13, 16, 2048])   # (12 / 13: the rotation goes from items of two outputs to four)
 def test_config4_down_projection(oracle, M):
     K, N = 17408, 5120
