@@ -297,7 +297,7 @@ __device__ __forceinline__ void paley_quantize(const float *buf, int s, int cr, 
     constexpr int NB = (NG + 15) / 16;     // batches of sixteen registers: batch b is delivered to the lanes of row b
     static_assert(NB <= 2, "two rows of lanes take the parameters");
     float x[NG];
-    int e0[NPAIR][2];   // element index of output 0 of the run's first column
+    int e_first = 0;   // element index of output 0 of the first run's first column; run r starts 64 r behind it
 #pragma unroll
     for (int pr = 0; pr < NPAIR; ++pr) {
         const int c0 = (cr + 2 * pr) * 64 + lane, c1 = c0 + 64;
@@ -313,8 +313,7 @@ __device__ __forceinline__ void paley_quantize(const float *buf, int s, int cr, 
             x[(2 * pr) * kOut + o] = out0[o] * scale;
             x[(2 * pr + 1) * kOut + o] = out1[o] * scale;
         }
-        e0[pr][0] = __builtin_amdgcn_readfirstlane(b0 + kOut * s * m);
-        e0[pr][1] = __builtin_amdgcn_readfirstlane(b1 + kOut * s * m);
+        if (pr == 0) e_first = __builtin_amdgcn_readfirstlane(b0 + kOut * s * m);
     }
     RQ_STAMP_AT(stamps, 9);
     RQ_STAMP_AT(stamps, 4);
@@ -370,15 +369,10 @@ __device__ __forceinline__ void paley_quantize(const float *buf, int s, int cr, 
     const float inv_l = 1.0f / ((float) mg_l * u);
     const float zf_l = fminf(fmaxf(rintf(-lo_l * inv_l), 0.0f), 15.0f);
     if (mine) {
-        // (group g: run g / kOut of the wavefront, output g % kOut)
+        // (group g: run g / kOut of the wavefront, output g % kOut; the wavefront's runs are neighbours in one rotation
+        // block, so run r starts 64 r elements behind run 0)
         const int run = g_l / kOut, o = g_l - run * kOut;
-        int e = e0[0][0];
-#pragma unroll
-        for (int pr = 0; pr < NPAIR; ++pr) {
-            if (run == 2 * pr) e = e0[pr][0];
-            if (run == 2 * pr + 1) e = e0[pr][1];
-        }
-        s_mz[(e + o * m) >> 6] = mg_l | ((8 - (int) zf_l) & 0xFF) << 8;
+        s_mz[(e_first >> 6) + run + o * (m >> 6)] = mg_l | ((8 - (int) zf_l) & 0xFF) << 8;
     }
     // (all code words first, then the stores under one lane mask: with a store per group in between, every group's
     // dependent chain ran alone, with the wait states of its lane permutations unfilled)
@@ -401,8 +395,7 @@ __device__ __forceinline__ void paley_quantize(const float *buf, int s, int cr, 
         uint32_t *dst = s_act + (lane >> 3);
 #pragma unroll
         for (int i = 0; i < NG; ++i) {
-            const int e = e0[i / (2 * kOut)][(i / kOut) & 1] + (i % kOut) * m;
-            dst[e >> 3] = word[i];
+            dst[(e_first >> 3) + 8 * (i / kOut) + (i % kOut) * (m >> 3)] = word[i];
         }
     }
     RQ_STAMP_AT(stamps, 12);
@@ -977,7 +970,7 @@ hipError_t launch_decode(const DecodeArgs &d, hipStream_t stream) {
         const int ncols = d.K / d.p, col_runs = ncols / 64, n_it = 4 * col_runs;
         const int per_wave = n_it / kRotWaves;
         if ((ncols & 63) == 0 && (d.m & 63) == 0 && n_it == per_wave * kRotWaves && (per_wave == 2 || per_wave == 4) &&
-            col_runs % per_wave == 0) {
+            col_runs % per_wave == 0 && (d.m / 64) % per_wave == 0) {   // (a wavefront's runs lie in one rotation block)
             paley_pairs = per_wave / 2;
         }
     }

@@ -364,12 +364,16 @@ __device__ __forceinline__ void load_row_fwht16(float *buf, const float *__restr
 // (reference lines 2454-2464). t - v is formed as t + (-v): the same IEEE operation.
 template <int CTRL>
 __device__ __forceinline__ void dpp_stage(float (&v)[16], uint32_t upper_sign) {
+    // (all sign flips first: taken value by value, every sum waited out the two wait states that an instruction with a
+    // lane permutation needs behind the write of any of its operands)
+    float sv[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) sv[j] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v[j]) ^ upper_sign);
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
         const float t = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v[j]), CTRL,
                                                                               0xF, 0xF, false));
-        const float sv = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v[j]) ^ upper_sign);
-        v[j] = t + sv;
+        v[j] = t + sv[j];
     }
 }
 
