@@ -516,7 +516,7 @@ def main():
                 roofline_m2048 = {"bound": "mfma", "achieved": round(ops / kms / 1e9, 1), "peak": INT8_PEAK_TOPS,
                                   "unit": "TOP/s", "frac": round(ops / kms / 1e9 / INT8_PEAK_TOPS, 4),
                                   "traffic": profiled_traffic_bytes(GEMM_PROFILE, "traffic_bytes_per_launch_m2048:"),
-                                  "kernel": "rq_gemm6_kernel<1> (fp6 MFMA; whole tiles and K slices of one launch)"
+                                  "kernel": "rq_gemm6_kernel<1, false> (fp6 MFMA; whole tiles and K slices of one launch)"
                                             if os.environ.get("RQ_GEMM_FP6", "1") != "0" else "rq_gemm_kernel (int8 MFMA)",
                                   "kernel_us": round(kms * 1e3, 3), "workload": "W4A4H K=5120 N=17408 M=2048",
                                   "op_us": extra[name]["op_us"], "op_tops": extra[name]["op_tops"],
