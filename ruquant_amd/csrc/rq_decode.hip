@@ -548,8 +548,10 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         bool waited = false;
 
         // remainder item `i` of this workgroup -> address of its 1 KiB (8 rows x 4 groups x 2 halves)
-        // (items past the end read the workgroup's own first KiB again, so that those reads spread over the memory
-        // channels like the real ones; a workgroup without remainder rows takes the remainder's first KiB: valid memory)
+        // (items past the end read the first 16 bytes of the workgroup's own first item, every lane the same: one
+        // request per load, and a different line for every workgroup; with the whole first KiB read again the load
+        // path carried up to as many KiB of these as of real items. A workgroup without remainder rows takes the
+        // remainder's first bytes: valid memory)
         auto tail_address = [&](int i, bool valid) -> const uint8_t * {
             const int ol = valid ? (int) (((uint32_t) i * (uint32_t) a.inv_nblk) >> 22) : 0;
             const int bb = valid ? i - ol * nblk : 0;
@@ -558,7 +560,7 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
             const int wsel = (panel >= a.ws.first[1]) + (panel >= a.ws.first[2]);
             const int wpanel = panel - (wsel == 0 ? 0 : wsel == 1 ? a.ws.first[1] : a.ws.first[2]);
             const uint8_t *codes = wsel == 0 ? a.ws.codes[0] : wsel == 1 ? a.ws.codes[1] : a.ws.codes[2];
-            return codes + ((size_t) wpanel * ng + 4 * bb) * 2048 + (o & 7) * 128 + lane_off;
+            return codes + ((size_t) wpanel * ng + 4 * bb) * 2048 + (o & 7) * 128 + (valid ? lane_off : 0u);
         };
         // the first round of remainder items goes out with the first round of the whole panels
         v4u wt[MT > 0 ? MT : 1];
@@ -889,14 +891,30 @@ hipError_t launch_pmt(const DecodeKernelArgs &k, int grid, size_t lds, hipStream
 }
 
 // whole panels: 10 groups per wavefront and round cover K = 5120 in one round (12: K = 6144); the remainder gets 4
-// items per wavefront and round beside whole panels, 12 when the launch is remainder only
+// items per wavefront and round beside whole panels, 12 to 26 (the smallest even count that holds them) when the launch is
+// remainder only
 template <int P>
 hipError_t launch_p(const DecodeKernelArgs &k, int grid, size_t lds, hipStream_t stream) {
     if (k.main_panels == 0) {
         // remainder only: all of a wavefront's items in flight when they are at most 26
-        const int octets = (k.q_base + (k.q_extra > 0 ? 1 : 0) + 1) / 2 + 1;   // most octets a run of quads touches
+        // most octets that a workgroup's run of quads touches (a run that starts or ends inside an octet shares it)
+        int octets = 0;
+        for (int s = 0; s < grid; ++s) {
+            const int q0 = s * k.q_base + (s < k.q_extra ? s : k.q_extra), q1 = q0 + k.q_base + (s < k.q_extra ? 1 : 0);
+            const int n = q1 > q0 ? ((q1 + 1) >> 1) - (q0 >> 1) : 0;
+            if (n > octets) octets = n;
+        }
         const int per_wave = (octets * (k.K / 256) + kStrWaves - 1) / kStrWaves;
-        if (per_wave > 12) return launch_pmt<P, 0, 26>(k, grid, lds, stream);
+        // The smallest form that holds them all: a slot too few is a second round of loads behind the first round's
+        // fold (K = 5120, N = 11264, 15 items: 8.4 -> 10.2 us with 14 slots), and every slot too many costs 0.1 us
+        // (N = 8192, 10 items: 6.9 us with 12 slots, 9.1 us with 26).
+        if (per_wave > 24) return launch_pmt<P, 0, 26>(k, grid, lds, stream);
+        if (per_wave > 22) return launch_pmt<P, 0, 24>(k, grid, lds, stream);
+        if (per_wave > 20) return launch_pmt<P, 0, 22>(k, grid, lds, stream);
+        if (per_wave > 18) return launch_pmt<P, 0, 20>(k, grid, lds, stream);
+        if (per_wave > 16) return launch_pmt<P, 0, 18>(k, grid, lds, stream);
+        if (per_wave > 14) return launch_pmt<P, 0, 16>(k, grid, lds, stream);
+        if (per_wave > 12) return launch_pmt<P, 0, 14>(k, grid, lds, stream);
         return launch_pmt<P, 0, 12>(k, grid, lds, stream);
     }
     const int gpw = (k.K / kGroup + kStrWaves - 1) / kStrWaves;
@@ -916,6 +934,12 @@ hipError_t allow_lds() {
 template <int P>
 hipError_t allow_lds_p() {
     hipError_t e = allow_lds<P, 0, 12>();
+    if (e == hipSuccess) e = allow_lds<P, 0, 14>();
+    if (e == hipSuccess) e = allow_lds<P, 0, 16>();
+    if (e == hipSuccess) e = allow_lds<P, 0, 18>();
+    if (e == hipSuccess) e = allow_lds<P, 0, 20>();
+    if (e == hipSuccess) e = allow_lds<P, 0, 22>();
+    if (e == hipSuccess) e = allow_lds<P, 0, 24>();
     if (e == hipSuccess) e = allow_lds<P, 0, 26>();
     if (e == hipSuccess) e = allow_lds<P, 10, 4>();
     if (e == hipSuccess) e = allow_lds<P, 10, 0>();
@@ -990,6 +1014,12 @@ hipError_t launch_decode(const DecodeArgs &d, hipStream_t stream) {
         grid += cus;
     }
     if (grid > n_panels * 16) grid = n_panels * 16;
+    // Fewer panels than compute units, but most of them: one whole panel per workgroup on n_panels compute units and
+    // the others idle. A panel streams as contiguous KiB with the lane as the row; rows dealt in quads over all
+    // compute units are read as 128-byte pieces, and that form loses from about 55 % of the compute units on
+    // (K = 5120: N = 8192 6.9 us in quads, 7.4 us in panels; N = 10240 7.7 and 7.55; N = 12288 8.5 and 8.0; N = 15360
+    // 10.3 and 8.6; N = 16320 10.7 and 8.9; K = 4096, where the panel is shorter: N = 12288 7.5 and 7.7).
+    if (grid == cus && n_panels < cus && n_panels * 8 >= cus * (d.K >= 5120 ? 5 : 7)) grid = n_panels;
     k.main_panels = n_panels / grid;
     k.tail_panel0 = k.main_panels * grid;
     const int tail_quads = (n_panels - k.tail_panel0) * 16;

@@ -416,6 +416,56 @@ def test_one_token_whole_panels(oracle, type_, K, N, n_rot, mult):
     assert bits_equal(got, want), first_mismatch(got, want)
 
 
+@pytest.mark.parametrize("type_,K,N,mult", [
+    (rq.TYPE_W4A4H, 5120, 10240, 0),     # 160 panels: the fewest that run as one whole panel per workgroup (K >= 5120)
+    (rq.TYPE_W4A4H, 5120, 16320, 64),    # 255 panels, weight multipliers per group
+    (rq.TYPE_W4A4H, 5120, 12000, 0),     # 187.5 panels: the last one is ragged
+    (rq.TYPE_W4A4H, 6144, 10304, 256),   # 161 panels of 12 groups per wavefront
+    (rq.TYPE_W4A4, 4096, 14400, 0),      # 225 panels of a shorter row (from 7/8 of the compute units on)
+    (rq.TYPE_W4A4H, 5120, 9216, 0),      # 144 panels: still dealt in quads, 14 items per wavefront in flight
+    (rq.TYPE_W4A4H, 5120, 7168, 0),      # 7 quads per workgroup (runs start inside octets)
+    (rq.TYPE_W4A4, 4096, 13056, 64),     # 204 panels of a shorter row, dealt in quads: 16 items in flight
+    (rq.TYPE_W4A4H, 10240, 4992, 0),     # long rows, few of them: 40 blocks per octet, 20 items in flight
+    (rq.TYPE_W4A4H, 16384, 4160, 0),     # two rounds of 26 items
+])
+def test_one_token_between_one_and_two_rounds_of_panels(oracle, type_, K, N, mult):
+    """One token against weights of fewer panels than compute units. From 5/8 of them on (7/8 for rows shorter than
+    5120) every workgroup takes one whole panel and the other compute units stay idle; below, the rows are dealt in
+    quads over all compute units, a wavefront's items all in flight in the smallest of the forms for 12, 14, ... 26
+    items that holds them."""
+    had = type_ == rq.TYPE_W4A4H
+    blocks = synth.random_weight_blocks(N, K, 31, type_, clip=0.9, n_rot=K if had else None)
+    rng = np.random.default_rng(17)
+    if mult == 256:
+        blocks["sum"] = ((1 << 30) | rng.integers(1, 16, size=blocks["sum"].shape)).astype(np.int32)
+    elif mult == 64:
+        k = rng.integers(1, 16, size=blocks["sum"].shape + (4,))
+        blocks["sum"] = ((3 << 29) | k[..., 0] | (k[..., 1] << 4) | (k[..., 2] << 8) | (k[..., 3] << 12)).astype(np.int32)
+    W = rq.W4A4Weight(blocks, type_, DEV)
+    x = synth.activations("outlier_channels", 1, K, 19)
+    got = run_gpu(W, x)
+    want = oracle.mul_mat(type_, blocks, x, W.clip, n_rot=K if had else 0)
+    assert bits_equal(got, want), first_mismatch(got, want)
+
+
+def test_one_token_fused_weights_as_whole_panels_on_fewer_workgroups(oracle):
+    """Three weights in one call whose panels together (96 + 16 + 56 = 168, the last one ragged) run as one whole panel
+    per workgroup: a workgroup finds its weight from the panel index."""
+    K, type_ = 5120, rq.TYPE_W4A4H
+    ws, bl = [], []
+    for i, N in enumerate([6144, 1024, 3560]):
+        b = synth.random_weight_blocks(N, K, 40 + i, type_, clip=0.9)
+        bl.append(b)
+        ws.append(rq.W4A4Weight(b, type_, DEV))
+    x = synth.activations("student_t4", 1, K, 23)
+    xd = torch.from_numpy(x).to(DEV)
+    outs = rq.mul_mat_fused(ws, xd)
+    torch.cuda.synchronize()
+    for b, w, o in zip(bl, ws, outs):
+        want = oracle.mul_mat(type_, b, x, w.clip, n_rot=K)
+        assert bits_equal(o.cpu().numpy(), want), first_mismatch(o.cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("K,n_rot", [(5120, 5120), (6144, 6144), (10240, 10240), (3072, 3072), (5120, 2560), (12288, 12288)])
 @pytest.mark.parametrize("row", ["zeros", "one_spike", "constant", "negative_constant", "signed_zeros", "alternating",
                                  "one_group_only", "tiny"])
