@@ -482,7 +482,7 @@ int rq_w4a4_prepare_inplace(void *w_blocks_dev, int64_t K, int64_t N, void *plan
     if (K <= 0 || K % RQ_BLOCK_CODES != 0 || K > RQ_MAX_K || N <= 0 || N > (int64_t) 1 << 24) return RQ_E_UNSUPPORTED;
     const PreparedLayout L = prepared_layout(K, N);
     // the sections up to the flag word must fit where the blocks are
-    if (L.off_flags + 256 > (size_t) N * (size_t) (K / RQ_BLOCK_CODES) * RQ_BLOCK_BYTES) return RQ_E_WORKSPACE;
+    if (L.off_flags + kFlagRegionBytes > (size_t) N * (size_t) (K / RQ_BLOCK_CODES) * RQ_BLOCK_BYTES) return RQ_E_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(w_blocks_dev) & 255) != 0 || (reinterpret_cast<uintptr_t>(staging_dev) & 255) != 0) return RQ_E_WORKSPACE;
     if (staging_bytes < inplace_staging_min(L)) return RQ_E_WORKSPACE;
     if (gemm_fp6_enabled()) {

@@ -44,6 +44,12 @@ constexpr int kGemvMaxTokens = 64;  // workspaces of up to this many tokens hold
 constexpr int kFrag6 = 1536;      // bytes of one 32 x 64 fp6 MFMA fragment
 constexpr int kRowTile6 = 256;    // rows of one tile of the fp6 plane
 
+// The flag region of a prepared weight: int 0 = the flag word (bit 0: some weight multiplier differs from 1), ints 2-3 =
+// the device address of the fp6 plane; behind these 256 bytes, kFlagReplicas copies of the flag word, one per 64-byte
+// line, for the one-token kernel, whose 2048 stream wavefronts would otherwise all read the one line.
+constexpr int kFlagReplicas = 32;
+constexpr size_t kFlagRegionBytes = 256 + 64 * kFlagReplicas;
+
 struct PreparedLayout {
     int64_t K, N;
     int     ng;        // K / 64
@@ -73,7 +79,7 @@ inline PreparedLayout prepared_layout(int64_t K, int64_t N) {
     L.off_kmul = off;
     off = align_up(off + (size_t) L.n_panels * L.ng * kPanelRows, 256);
     L.off_flags = off;
-    off = align_up(off + 256, 256);
+    off = align_up(off + kFlagRegionBytes, 256);
     L.off_w6 = 0;
     if (gemm_fp6_enabled()) {
         L.off_w6 = off;

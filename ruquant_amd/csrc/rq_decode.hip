@@ -536,9 +536,13 @@ __global__ void __launch_bounds__(kDecThreads) rq_decode_kernel(const DecodeKern
         const int r8 = lane & 7, h = (lane >> 3) & 1, g4 = lane >> 4;
         const uint32_t lane_off = (uint32_t) (g4 * 2048 + h * 1024 + r8 * 16);
         // flag words of the weights (bit 0: some weight multiplier differs from 1)
-        const int32_t f0 = __builtin_nontemporal_load(a.ws.flags[0]);
-        const int32_t f1 = __builtin_nontemporal_load(a.ws.flags[1]);
-        const int32_t f2 = __builtin_nontemporal_load(a.ws.flags[2]);
+        // (from the copy of this workgroup's turn: with all 2048 stream wavefronts of a launch on the one line of the
+        // word itself, these loads, which sit in every wavefront's queue in front of most of its weights, took long to
+        // come back, and loads come back in order: K = 5120, N = 17408 9.72 -> 9.55 us, N = 12288 7.98 -> 7.72)
+        const int flag_copy = 64 + 16 * (int) (blockIdx.x % kFlagReplicas);
+        const int32_t f0 = __builtin_nontemporal_load(a.ws.flags[0] + flag_copy);
+        const int32_t f1 = __builtin_nontemporal_load(a.ws.flags[1] + flag_copy);
+        const int32_t f2 = __builtin_nontemporal_load(a.ws.flags[2] + flag_copy);
 
         RQ_STAMP(1);
 

@@ -89,11 +89,12 @@ __global__ void __launch_bounds__(256) rq_prepare6_kernel(const rq_block_w4a4 *_
 // the flag word of a prepared weight and, beside it, the device address of its fp6 plane (0: none), which the fp6
 // GEMM reads from here: the plane may live inside the prepared buffer or, for a weight prepared in place, elsewhere
 __global__ void rq_finish_flags_kernel(int32_t *flags, const int32_t *from, const uint8_t *plane6) {
+    const int32_t f = from ? from[0] : flags[0];
     if (threadIdx.x == 0) {
-        const int32_t f = from ? from[0] : flags[0];
         flags[0] = f;
         *reinterpret_cast<unsigned long long *>(flags + 2) = (unsigned long long) (uintptr_t) plane6;
     }
+    if (threadIdx.x < kFlagReplicas) flags[64 + 16 * threadIdx.x] = f;   // (the copies: a 64-byte line each)
 }
 
 }  // namespace
